@@ -1,0 +1,181 @@
+/*
+ * paraattn_hip.h -- C ABI of libparaattn_hip.so (gfx950 / MI355X).
+ *
+ * The reference (chengzeyi/ParaAttention) is pure Python: its attention ops end
+ * in aten CUDA kernels and it has no FFI of its own.  This header is therefore
+ * the binding surface a maintainer would target from the reference's op layer;
+ * every entry point names the reference interface it stands in for.
+ *
+ * Conventions
+ *  - All pointers are device pointers unless the name ends in _host.
+ *  - Nothing here allocates or frees device memory and nothing synchronises:
+ *    work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ *    null stream) and the call returns at once.  Outputs and workspaces belong
+ *    to the caller and must stay alive until the stream work has run.
+ *  - Functions return PA_OK (0) or a negative PA_ERR_* code and never throw or
+ *    exit; pa_last_error() gives the text for the calling thread.
+ *  - Strides are in elements.  The innermost (head_dim) stride must be 1.
+ */
+#ifndef PARAATTN_HIP_H
+#define PARAATTN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* exported symbol (the library is built with hidden default visibility) */
+#define PA_API __attribute__((visibility("default")))
+
+#define PA_OK 0
+#define PA_ERR_INVALID (-1)     /* bad argument (null pointer, negative size ...) */
+#define PA_ERR_UNSUPPORTED (-2) /* shape / dtype / stride the kernels do not cover */
+#define PA_ERR_LAUNCH (-3)      /* HIP reported an error at launch */
+#define PA_ERR_WORKSPACE (-4)   /* workspace too small */
+
+/* element types of activations */
+#define PA_DTYPE_BF16 0
+#define PA_DTYPE_F16 1
+#define PA_DTYPE_F32 2
+
+/* ABI version of this header (bumped on any signature change). */
+PA_API int pa_abi_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+PA_API const char* pa_last_error(void);
+
+/*
+ * Dense non-causal scaled-dot-product attention forward.
+ *   out[b,h,i,:] = softmax_j(scale * q[b,h,i,:].k[b,h,j,:]) @ v[b,h,j,:]
+ *   lse[b,h,i]   = log sum_j exp(scale * q.k)      (natural log, fp32)
+ * Stands in for para_attn.ops.attention_forward_with_lse
+ * (src/para_attn/ops/__init__.py:112-179: the aten flash / efficient / cuDNN
+ * forward + [:2]) and, with lse == NULL, for para_attn.ops.attention_forward
+ * (src/para_attn/ops/__init__.py:204-223).
+ *
+ * q [B,H,Sq,D], k,v [B,H,Skv,D], out [B,H,Sq,D]: dtype bf16 or f16, strides
+ * {batch, head, seq} in elements, head_dim stride 1, every row start 16-byte
+ * aligned.  lse: contiguous fp32 [B,H,Sq] or NULL.  D == 128 (or 64).
+ * kv_len: NULL, or int32 [B] device array giving, per batch element, how many
+ * leading keys take part (the rest are ignored); this is how the sparse_kv op
+ * (src/para_attn/ops/__init__.py:248-299) runs once its mask is a prefix.
+ */
+PA_API int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* out, float* lse,
+                    int dtype, int B, int H, int Sq, int Skv, int D,
+                    const int64_t q_strides[3], const int64_t k_strides[3],
+                    const int64_t v_strides[3], const int64_t out_strides[3],
+                    float scale, const int32_t* kv_len, void* stream);
+
+/*
+ * Block-sparse attention forward: query block i (of q_block rows, counted from
+ * q_lo) attends key block j (of kv_block rows, counted from kv_lo) iff
+ * block_mask[hm,i,j] != 0; query rows outside [q_lo, q_lo + nQ*q_block) attend
+ * every key, and keys outside [kv_lo, kv_lo + nK*kv_block) are attended by every
+ * query.  Equals dense attention with -inf on the dropped tiles.  Replaces the
+ * Python loop of para_attn.sparse_attn.StructuredSparseAttnFunc.forward
+ * (src/para_attn/sparse_attn.py:74-278: one SDPA launch per run of kept blocks
+ * plus one merge each).  Unlike the reference it also returns the LSE.
+ *
+ * block_mask: uint8 [Hm,nQ,nK] contiguous, Hm == 1 (shared by all heads, the
+ * reference's 2-D mask, sparse_attn.py:107) or Hm == H.
+ * runs_ws: int32 workspace of at least pa_blocksparse_workspace_bytes() bytes;
+ * it receives, per (hm, query segment), the list of key ranges the kernel
+ * walks (the mask's runs of kept blocks, merged, exactly as
+ * sparse_attn.py:215-234 scans them).
+ * A query block that keeps no key at all yields out = 0 and lse = -inf.
+ */
+PA_API int pa_attn_fwd_blocksparse(const void* q, const void* k, const void* v, void* out, float* lse,
+                            int dtype, int B, int H, int Sq, int Skv, int D,
+                            const int64_t q_strides[3], const int64_t k_strides[3],
+                            const int64_t v_strides[3], const int64_t out_strides[3],
+                            float scale, const uint8_t* block_mask, int Hm, int nQ, int nK,
+                            int q_lo, int q_block, int kv_lo, int kv_block,
+                            int32_t* runs_ws, size_t runs_ws_bytes, void* stream);
+
+/* Bytes of runs_ws needed by pa_attn_fwd_blocksparse for a [Hm,nQ,nK] mask. */
+PA_API size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK);
+
+/*
+ * Only the run extraction of pa_attn_fwd_blocksparse (for tests and for callers
+ * that reuse one mask over many calls).  Layout of runs_ws, with
+ * nSeg = nQ + 2 (segment 0 = rows left of q_lo, 1..nQ = mask rows, nQ+1 = rows
+ * right of the sparse range) and cap = nK/2 + 3:
+ *   int32 count[Hm*nSeg], then int32 range[Hm*nSeg][cap][2] as {begin,end} key
+ *   indices in ascending order.
+ */
+PA_API int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int nQ, int nK, int Skv,
+                              int kv_lo, int kv_block, int32_t* runs_ws, size_t runs_ws_bytes,
+                              void* stream);
+
+/*
+ * One step of the ring-attention partial-result merge, fused into one pass:
+ *   w       = sigmoid(blk_lse - acc_lse)
+ *   out     = acc_out - w * (acc_out - blk_out)
+ *   lse_out = acc_lse - logsigmoid(acc_lse - blk_lse)
+ * i.e. torch's _SDPAMerger._merge_one (torch/distributed/tensor/experimental/
+ * _context_parallel/_attention.py:150-203, the arithmetic the reference drives
+ * from src/para_attn/para_attn_interface.py:182-193 and
+ * src/para_attn/sparse_attn.py:174-259), computed in fp32.
+ *
+ * acc_out [rows,D] (acc_dtype), blk_out [rows,D] (blk_dtype), out [rows,D]
+ * (out_dtype), all contiguous; acc_lse, blk_lse, lse_out fp32 [rows].  out may
+ * alias acc_out when the dtypes match and lse_out may alias acc_lse (in-place
+ * step).  Choosing acc_dtype = bf16 folds the merger's first-step cast
+ * (_attention.py:209-211) into the step, out_dtype = bf16 folds results()'s
+ * final cast (_attention.py:215-223).  D must be a multiple of 8.
+ */
+PA_API int pa_merge_lse(const void* acc_out, int acc_dtype, const float* acc_lse,
+                 const void* blk_out, int blk_dtype, const float* blk_lse,
+                 void* out, int out_dtype, float* lse_out,
+                 int64_t rows, int D, void* stream);
+
+/*
+ * First Block Cache residual-difference reduction:
+ *   mean_diff = mean(|prev - cur|), mean_prev = mean(|prev|), ratio = mean_diff / mean_prev
+ * with torch's rounding chain for the activation dtype: the difference is
+ * rounded to the dtype per element, both means are rounded to the dtype once,
+ * and the quotient is rounded to the dtype.  Stands in for the seven torch ops
+ * of are_two_tensors_similar (src/para_attn/first_block_cache/utils.py:228-233);
+ * the caller keeps `.item() < threshold` (utils.py:234).
+ *
+ * prev, cur: [n_rows, row_len] views; *_row_stride and *_col_stride in
+ * elements (col stride > 1 covers the [..., ::downsample_factor] slice of
+ * utils.py:276-278).  ratio_out: one element of `dtype`.  stats_out: NULL or
+ * fp32[2] receiving {mean_diff, mean_prev} after rounding to dtype.
+ * workspace: at least pa_fbcache_workspace_bytes() bytes, any contents.
+ */
+PA_API int pa_fbcache_absdiff_ratio(const void* prev, const void* cur, int dtype,
+                             int64_t n_rows, int64_t row_len,
+                             int64_t prev_row_stride, int64_t prev_col_stride,
+                             int64_t cur_row_stride, int64_t cur_col_stride,
+                             void* ratio_out, float* stats_out,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+PA_API size_t pa_fbcache_workspace_bytes(void);
+
+/*
+ * Fused first-block residual + reduction (neighbours of the reduction in
+ * CachedTransformerBlocks.forward, src/para_attn/first_block_cache/utils.py:359-366):
+ *   resid = hidden - hidden0      (rounded to dtype, written to resid_out)
+ *   ratio as above with cur = resid
+ * All tensors contiguous with n elements.  prev may be NULL (first step: only
+ * the residual is written, ratio_out is left untouched).
+ */
+PA_API int pa_fbcache_residual_ratio(const void* hidden, const void* hidden0, const void* prev,
+                              void* resid_out, int dtype, int64_t n,
+                              void* ratio_out, float* stats_out,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Cache-hit path: out = resid + hidden (src/para_attn/first_block_cache/utils.py:237-259),
+ * contiguous, n elements, rounded to dtype.  out may alias hidden.
+ */
+PA_API int pa_fbcache_apply_residual(const void* resid, const void* hidden, void* out, int dtype,
+                              int64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PARAATTN_HIP_H */

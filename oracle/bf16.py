@@ -1,0 +1,25 @@
+"""Round-to-nearest-even bf16 / fp16 rounding in numpy (test infrastructure)."""
+import numpy as np
+
+
+def round_bf16(x):
+    """fp32 array -> nearest bf16 value, returned as fp32 (ties to even, NaN kept)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    bias = ((u >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF)
+    r = ((u + bias) & np.uint32(0xFFFF0000)).view(np.float32)
+    return np.where(np.isnan(x), x, r).astype(np.float32)
+
+
+def round_f16(x):
+    return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def round_to(x, dtype_name):
+    if dtype_name == "bf16":
+        return round_bf16(x)
+    if dtype_name == "f16":
+        return round_f16(x)
+    if dtype_name == "f32":
+        return np.asarray(x, dtype=np.float32)
+    raise ValueError(dtype_name)

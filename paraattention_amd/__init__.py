@@ -1,0 +1,16 @@
+"""paraattention_amd: the attention op layer of ParaAttention for MI355X (gfx950).
+
+Importing the package registers the ``torch.ops.para_attn.*`` operators; the HIP
+library itself is loaded on first use and its absence is an error, not a
+fallback.
+"""
+from . import config  # noqa: F401
+from . import ops  # noqa: F401  (registers torch.ops.para_attn.*)
+from . import fbcache, merge, sparse  # noqa: F401
+from .merge import SDPAMerger, ring_sweep  # noqa: F401
+from .sparse import StructSparseAttnMode, struct_sparse_attn_func  # noqa: F401
+
+__all__ = [
+    "config", "ops", "merge", "sparse", "fbcache",
+    "SDPAMerger", "ring_sweep", "StructSparseAttnMode", "struct_sparse_attn_func",
+]

@@ -1,0 +1,591 @@
+// Non-causal attention forward (output + fp32 log-sum-exp) for gfx950.
+//
+// One workgroup = 4 wavefronts = 128 query rows; each wavefront owns 32 query
+// rows for the whole key sweep.  Keys/values stream through LDS in tiles of 64
+// rows, double buffered (global -> registers one tile ahead -> LDS).
+//
+// Both GEMMs run transposed so that the softmax needs no cross-lane traffic and
+// P never leaves registers:
+//   S^T[n,m] = sum_d K[n,d] Q[m,d]     A = K tile (LDS), B = Q (registers)
+//   O^T[d,m] = sum_n V^T[d,n] P^T[n,m] A = V^T tile (LDS, transposed on the way
+//                                      in), B = P^T = the S^T accumulators,
+//                                      exponentiated and packed to 16 bit
+// With v_mfma_f32_32x32x16 the accumulator of lane (m = lane%32, h = lane/32)
+// holds rows n = 8a + 4h + b (a,b = 0..3) of column m, so a query row's 32
+// scores of a sub-tile sit in two lanes (reduction = 1 swap), and accumulator
+// registers 8c..8c+7 are exactly the 8 contraction slots lane (m,h) must supply
+// as B operand of the second GEMM, provided V^T is laid out in LDS with the
+// matching permutation of n (bits 2 and 3 of n swapped).
+//
+// Stands in for the aten flash/efficient/cuDNN forward kernels the reference
+// dispatches to (src/para_attn/ops/__init__.py:48-157) and, with a list of key
+// ranges per query segment, for the run loop of the reference's block-sparse
+// mode (src/para_attn/sparse_attn.py:209-240).
+
+#include "pa_common.h"
+
+namespace pa {
+
+constexpr int BM = 128;       // query rows per workgroup
+constexpr int BN = 64;        // key rows per LDS tile
+constexpr int NTHREADS = 256;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+// The running maximum is only raised when a tile exceeds it by more than this
+// many powers of two; below that the accumulators keep their scale (P <= 2^8).
+constexpr float RESCALE_SLACK = 8.0f;
+
+struct AttnParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;
+  int B, H, Sq, Skv;
+  int64_t qs_b, qs_h, qs_s;
+  int64_t ks_b, ks_h, ks_s;
+  int64_t vs_b, vs_h, vs_s;
+  int64_t os_b, os_h, os_s;
+  float scale_log2;  // scale * log2(e), > 0
+  int n_qtiles;      // workgroups per (batch, head)
+  const int32_t* kv_len;  // dense: optional per-batch key count
+  // block-sparse only
+  const int32_t* runs;  // count[Hm*nSeg] then range[Hm*nSeg][cap][2]
+  int Hm, nQ, cap;
+  int q_lo, q_block;
+  int tiles_left, tiles_per_block;
+};
+
+template <int D>
+struct Smem {
+  static constexpr int KSTRIDE = D + 8;    // elements; +16 B keeps b128 reads conflict free
+  static constexpr int VSTRIDE = BN + 8;   // V^T row: 64 keys + 16 B pad
+  static constexpr int K_ELEMS = BN * KSTRIDE;
+  static constexpr int V_ELEMS = D * VSTRIDE;
+  static constexpr int BYTES = 2 * (K_ELEMS + V_ELEMS) * 2;
+};
+
+// Key tiles of one workgroup: walks a list of [begin,end) ranges in steps of BN.
+struct TileIter {
+  const int32_t* ranges;  // pairs
+  int nranges;
+  int ri;
+  int pos, end;
+  int one[2];  // storage for the single dense range
+  __device__ __forceinline__ void init_dense(int len) {
+    one[0] = 0;
+    one[1] = len;
+    ranges = nullptr;
+    nranges = len > 0 ? 1 : 0;
+    ri = 0;
+    pos = 0;
+    end = len;
+  }
+  __device__ __forceinline__ void init_list(const int32_t* r, int n) {
+    ranges = r;
+    nranges = n;
+    ri = 0;
+    if (n > 0) {
+      pos = r[0];
+      end = r[1];
+    } else {
+      pos = end = 0;
+    }
+  }
+  __device__ __forceinline__ bool valid() const { return ri < nranges; }
+  // current tile: rows [n0, n0 + nvalid), clamp row index to last
+  __device__ __forceinline__ void get(int& n0, int& nvalid) const {
+    n0 = pos;
+    int left = end - pos;
+    nvalid = left < BN ? left : BN;
+  }
+  __device__ __forceinline__ void next() {
+    pos += BN;
+    if (pos >= end) {
+      ++ri;
+      if (ri < nranges) {
+        pos = ranges[2 * ri];
+        end = ranges[2 * ri + 1];
+      }
+    }
+  }
+};
+
+template <typename T, int D, bool SPARSE>
+__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+  typedef typename T::vec8 vec8;
+  typedef Smem<D> SM;
+  constexpr int DC = D / 16;   // contraction chunks of the first GEMM
+  constexpr int DB = D / 32;   // 32-row blocks of O^T
+  constexpr int CH = D / 8;    // 16-byte chunks per K/V row
+  constexpr int KROWS_PER_PASS = NTHREADS / CH;
+  constexpr int KPASSES = BN / KROWS_PER_PASS;
+  constexpr int VGROUPS = BN / 4;  // groups of 4 key rows
+  constexpr bool V_ALL_THREADS = (NTHREADS / CH) == VGROUPS;
+  static_assert(NTHREADS / CH >= VGROUPS, "V loader mapping");
+
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* sK = smem;                        // [2][BN][KSTRIDE]
+  uint16_t* sV = smem + 2 * SM::K_ELEMS;      // [2][D][VSTRIDE]  (V^T, keys permuted)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  // ---- which query rows ------------------------------------------------------
+  const int qt = blockIdx.x % p.n_qtiles;
+  const int bh = blockIdx.x / p.n_qtiles;
+  const int head = bh % p.H;
+  const int batch = bh / p.H;
+
+  int row_begin, row_end;  // query rows [row_begin, row_end) of this workgroup
+  TileIter it;
+  if constexpr (SPARSE) {
+    int seg, tin;
+    if (qt < p.tiles_left) {
+      seg = 0;
+      tin = qt;
+      row_begin = tin * BM;
+      row_end = p.q_lo;
+    } else {
+      int r = qt - p.tiles_left;
+      int blk = r / p.tiles_per_block;
+      if (blk < p.nQ) {
+        seg = 1 + blk;
+        tin = r - blk * p.tiles_per_block;
+        row_begin = p.q_lo + blk * p.q_block + tin * BM;
+        row_end = p.q_lo + (blk + 1) * p.q_block;
+      } else {
+        seg = p.nQ + 1;
+        tin = r - p.nQ * p.tiles_per_block;
+        row_begin = p.q_lo + p.nQ * p.q_block + tin * BM;
+        row_end = p.Sq;
+      }
+    }
+    if (row_end > row_begin + BM) row_end = row_begin + BM;
+    const int nseg = p.nQ + 2;
+    const int hm = p.Hm == 1 ? 0 : head;
+    const int sidx = hm * nseg + seg;
+    const int cnt = p.runs[sidx];
+    it.init_list(p.runs + (size_t)p.Hm * nseg + (size_t)sidx * p.cap * 2, cnt);
+  } else {
+    row_begin = qt * BM;
+    row_end = row_begin + BM < p.Sq ? row_begin + BM : p.Sq;
+    int len = p.Skv;
+    if (p.kv_len) {
+      int kl = p.kv_len[batch];
+      len = kl < len ? (kl < 0 ? 0 : kl) : len;
+    }
+    it.init_dense(len);
+  }
+
+  const uint16_t* qbase = (const uint16_t*)p.q + batch * p.qs_b + head * p.qs_h;
+  const uint16_t* kbase = (const uint16_t*)p.k + batch * p.ks_b + head * p.ks_h;
+  const uint16_t* vbase = (const uint16_t*)p.v + batch * p.vs_b + head * p.vs_h;
+
+  // ---- Q fragment: B operand of the first GEMM, kept for the whole sweep -----
+  const int my_row = row_begin + wave * 32 + l32;
+  const bool row_ok = my_row < row_end;
+  vec8 qf[DC];
+  {
+    int r = row_ok ? my_row : (row_end - 1);
+    const uint16_t* qp = qbase + (int64_t)r * p.qs_s + 8 * hh;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
+  }
+
+  // ---- global -> register staging of one K/V tile ----------------------------
+  u32x4 kreg[KPASSES];
+  u32x4 vreg[4];
+  const int k_chunk = tid % CH;
+  const int k_row0 = tid / CH;
+  const int v_dcol = tid % CH;
+  const int v_grp = tid / CH;  // group of 4 key rows
+  const bool v_active = V_ALL_THREADS || v_grp < VGROUPS;
+  // position of the group inside V^T rows: swap the two low bits of the group
+  const int v_grp_perm = (v_grp & ~3) | ((v_grp & 1) << 1) | ((v_grp >> 1) & 1);
+
+  auto load_tile = [&](int n0, int nvalid) {
+    const int last = n0 + nvalid - 1;
+#pragma unroll
+    for (int i = 0; i < KPASSES; ++i) {
+      int r = n0 + k_row0 + i * KROWS_PER_PASS;
+      r = r < last ? r : last;
+      kreg[i] = *(const u32x4*)(kbase + (int64_t)r * p.ks_s + 8 * k_chunk);
+    }
+    if (v_active) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int r = n0 + 4 * v_grp + i;
+        r = r < last ? r : last;
+        vreg[i] = *(const u32x4*)(vbase + (int64_t)r * p.vs_s + 8 * v_dcol);
+      }
+    }
+  };
+
+  auto store_tile = [&](int buf) {
+    uint16_t* dK = sK + buf * SM::K_ELEMS;
+    uint16_t* dV = sV + buf * SM::V_ELEMS;
+#pragma unroll
+    for (int i = 0; i < KPASSES; ++i) {
+      int r = k_row0 + i * KROWS_PER_PASS;
+      *(u32x4*)(dK + r * SM::KSTRIDE + 8 * k_chunk) = kreg[i];
+    }
+    if (v_active) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int w = j >> 1;
+        const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+        u32x2 t;
+        t[0] = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
+        t[1] = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
+        *(u32x2*)(dV + (8 * v_dcol + j) * SM::VSTRIDE + 4 * v_grp_perm) = t;
+      }
+    }
+  };
+
+  // ---- accumulators -----------------------------------------------------------
+  floatx16 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m_run = -INFINITY;  // running maximum, in units of log2 (scaled scores)
+  float l_run = 0.f;        // this lane's share of the running sum
+  const float c = p.scale_log2;
+
+  // ---- pipeline prologue ------------------------------------------------------
+  int n0 = 0, nvalid = 0;
+  bool have = it.valid();
+  if (have) {
+    it.get(n0, nvalid);
+    load_tile(n0, nvalid);
+    it.next();
+    store_tile(0);
+  }
+  int cur_valid = nvalid;
+  bool have_next = it.valid();
+  int next_valid = 0;
+  if (have_next) {
+    it.get(n0, nvalid);
+    next_valid = nvalid;
+    load_tile(n0, nvalid);
+    it.next();
+  }
+  __syncthreads();
+
+  int buf = 0;
+  while (have) {
+    // registers hold tile j+1: park it in the other buffer, then fetch tile j+2
+    bool have_next2 = false;
+    int next2_valid = 0;
+    if (have_next) {
+      store_tile(buf ^ 1);
+      have_next2 = it.valid();
+      if (have_next2) {
+        it.get(n0, nvalid);
+        next2_valid = nvalid;
+        load_tile(n0, nvalid);
+        it.next();
+      }
+    }
+
+    const uint16_t* tK = sK + buf * SM::K_ELEMS;
+    const uint16_t* tV = sV + buf * SM::V_ELEMS;
+
+    // ---- S^T = K Q^T -----------------------------------------------------------
+    floatx16 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        vec8 a = *(const vec8*)(tK + (32 * t + l32) * SM::KSTRIDE + 16 * dc + 8 * hh);
+        s[t] = T::mfma32(a, qf[dc], s[t]);
+      }
+    }
+
+    // ---- mask the ragged end of a range ---------------------------------------
+    if (cur_valid < BN) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          int n = 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
+          if (n >= cur_valid) s[t][r] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax (row = lane%32, spread over the two half-waves) -------
+    float mx = s[0][0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[0][r]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[1][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float mx_s = mx * c;
+    if (__any(mx_s > m_run + RESCALE_SLACK)) {
+      const float m_new = fmaxf(m_run, mx_s);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+      m_run = m_new;
+    }
+    uint32_t pk[2][8];
+    float lsum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], c, -m_run));
+        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], c, -m_run));
+        lsum += p0 + p1;
+        pk[t][r >> 1] = T::pack2(p0, p1);
+      }
+    l_run += lsum;
+
+    // ---- O^T += V^T P^T ---------------------------------------------------------
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        u32x4 bw = {pk[t][4 * cc], pk[t][4 * cc + 1], pk[t][4 * cc + 2], pk[t][4 * cc + 3]};
+        vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          vec8 a = *(const vec8*)(tV + (32 * db + l32) * SM::VSTRIDE + 32 * t + 16 * cc + 8 * hh);
+          o[db] = T::mfma32(a, bfrag, o[db]);
+        }
+      }
+
+    __syncthreads();
+    buf ^= 1;
+    have = have_next;
+    cur_valid = next_valid;
+    have_next = have_next2;
+    next_valid = next2_valid;
+  }
+
+  // ---- epilogue -----------------------------------------------------------------
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  if (row_ok) {
+    uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)my_row * p.os_s;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        u32x2 w;
+        w[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
+        w[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
+        *(u32x2*)(op + 32 * db + 8 * a + 4 * hh) = w;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      p.lse[((int64_t)batch * p.H + head) * p.Sq + my_row] = lse;
+    }
+  }
+}
+
+// Turns a [Hm,nQ,nK] block mask into per-segment lists of key ranges.
+// One thread per (hm, segment); segments 0 and nQ+1 are the dense margins.
+__global__ void build_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK, int Skv,
+                                  int kv_lo, int kv_block, int cap, int32_t* ws) {
+  const int nseg = nQ + 2;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= Hm * nseg) return;
+  const int hm = idx / nseg;
+  const int seg = idx % nseg;
+  int32_t* cnt = ws + idx;
+  int32_t* rg = ws + (size_t)Hm * nseg + (size_t)idx * cap * 2;
+  int n = 0;
+  if (seg == 0 || seg == nQ + 1) {
+    if (Skv > 0) {
+      rg[0] = 0;
+      rg[1] = Skv;
+      n = 1;
+    }
+    *cnt = n;
+    return;
+  }
+  const uint8_t* row = mask + ((size_t)hm * nQ + (seg - 1)) * nK;
+  const int kv_hi = kv_lo + nK * kv_block;
+  int cur_b = -1, cur_e = -1;  // open range
+  auto push = [&](int b, int e) {
+    if (e <= b) return;
+    if (cur_e == b) {
+      cur_e = e;  // touches the open range: extend it
+    } else {
+      if (cur_e > cur_b) {
+        rg[2 * n] = cur_b;
+        rg[2 * n + 1] = cur_e;
+        ++n;
+      }
+      cur_b = b;
+      cur_e = e;
+    }
+  };
+  push(0, kv_lo);
+  int j = 0;
+  while (j < nK) {
+    if (!row[j]) {
+      ++j;
+      continue;
+    }
+    int e = j + 1;
+    while (e < nK && row[e]) ++e;
+    push(kv_lo + j * kv_block, kv_lo + e * kv_block);
+    j = e;
+  }
+  push(kv_hi, Skv);
+  if (cur_e > cur_b) {
+    rg[2 * n] = cur_b;
+    rg[2 * n + 1] = cur_e;
+    ++n;
+  }
+  *cnt = n;
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+static int check_common(const void* q, const void* k, const void* v, void* out, int dtype, int B,
+                        int H, int Sq, int Skv, int D, const int64_t* qs, const int64_t* ks,
+                        const int64_t* vs, const int64_t* os, float scale) {
+  if (!q || !k || !v || !out || !qs || !ks || !vs || !os) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  if (B < 0 || H < 0 || Sq < 0 || Skv < 0) PA_FAIL(PA_ERR_INVALID, "negative size");
+  if (dtype != PA_DTYPE_BF16 && dtype != PA_DTYPE_F16)
+    PA_FAIL(PA_ERR_UNSUPPORTED, "attention dtype must be bf16 or f16 (got code %d)", dtype);
+  if (D != 128 && D != 64) PA_FAIL(PA_ERR_UNSUPPORTED, "head_dim %d not supported (64 or 128)", D);
+  if (!(scale > 0.f) || !(scale < INFINITY)) PA_FAIL(PA_ERR_UNSUPPORTED, "scale must be positive and finite");
+  const int64_t* st[4] = {qs, ks, vs, os};
+  const void* ptr[4] = {q, k, v, out};
+  const char* nm[4] = {"query", "key", "value", "out"};
+  for (int i = 0; i < 4; ++i) {
+    if (((uintptr_t)ptr[i]) % 16) PA_FAIL(PA_ERR_UNSUPPORTED, "%s pointer not 16-byte aligned", nm[i]);
+    for (int j = 0; j < 3; ++j) {
+      if (st[i][j] < 0) PA_FAIL(PA_ERR_UNSUPPORTED, "%s has a negative stride", nm[i]);
+      if (st[i][j] % 8) PA_FAIL(PA_ERR_UNSUPPORTED, "%s stride %lld not a multiple of 8 elements", nm[i], (long long)st[i][j]);
+    }
+  }
+  if ((int64_t)B * H * ((Sq + BM - 1) / BM + 2) > 0x7fffffffLL) PA_FAIL(PA_ERR_UNSUPPORTED, "grid too large");
+  return PA_OK;
+}
+
+static void fill_params(AttnParams& p, const void* q, const void* k, const void* v, void* out,
+                        float* lse, int B, int H, int Sq, int Skv, const int64_t* qs,
+                        const int64_t* ks, const int64_t* vs, const int64_t* os, float scale) {
+  p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
+  p.B = B; p.H = H; p.Sq = Sq; p.Skv = Skv;
+  p.qs_b = qs[0]; p.qs_h = qs[1]; p.qs_s = qs[2];
+  p.ks_b = ks[0]; p.ks_h = ks[1]; p.ks_s = ks[2];
+  p.vs_b = vs[0]; p.vs_h = vs[1]; p.vs_s = vs[2];
+  p.os_b = os[0]; p.os_h = os[1]; p.os_s = os[2];
+  p.scale_log2 = scale * LOG2E;
+  p.kv_len = nullptr;
+  p.runs = nullptr;
+  p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.tiles_left = 0; p.tiles_per_block = 0;
+}
+
+template <typename T, int D, bool SPARSE>
+static int launch_attn(const AttnParams& p, hipStream_t stream) {
+  const size_t smem = Smem<D>::BYTES;
+  static bool attr_done = false;  // benign race: the call is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, SPARSE>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    attr_done = true;
+  }
+  const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
+  if (nblocks == 0) return PA_OK;
+  hipLaunchKernelGGL((attn_fwd_kernel<T, D, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem,
+                     stream, p);
+  PA_CHECK_LAUNCH("attn_fwd_kernel");
+  return PA_OK;
+}
+
+template <bool SPARSE>
+static int dispatch_attn(const AttnParams& p, int dtype, int D, hipStream_t stream) {
+  if (dtype == PA_DTYPE_BF16) {
+    if (D == 128) return launch_attn<BF16, 128, SPARSE>(p, stream);
+    return launch_attn<BF16, 64, SPARSE>(p, stream);
+  }
+  if (D == 128) return launch_attn<F16, 128, SPARSE>(p, stream);
+  return launch_attn<F16, 64, SPARSE>(p, stream);
+}
+
+extern "C" int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* out, float* lse,
+                               int dtype, int B, int H, int Sq, int Skv, int D,
+                               const int64_t q_strides[3], const int64_t k_strides[3],
+                               const int64_t v_strides[3], const int64_t out_strides[3],
+                               float scale, const int32_t* kv_len, void* stream) {
+  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                        out_strides, scale);
+  if (rc) return rc;
+  AttnParams p;
+  fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
+  p.kv_len = kv_len;
+  p.n_qtiles = (Sq + BM - 1) / BM;
+  return dispatch_attn<false>(p, dtype, D, (hipStream_t)stream);
+}
+
+extern "C" size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK) {
+  if (Hm <= 0 || nQ <= 0 || nK <= 0) return 0;
+  const size_t nseg = (size_t)nQ + 2;
+  const size_t cap = (size_t)nK / 2 + 3;
+  return sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2);
+}
+
+extern "C" int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int nQ, int nK, int Skv,
+                                         int kv_lo, int kv_block, int32_t* runs_ws,
+                                         size_t runs_ws_bytes, void* stream) {
+  if (!block_mask || !runs_ws) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  if (Hm <= 0 || nQ <= 0 || nK <= 0 || kv_block <= 0 || kv_lo < 0 || Skv < 0)
+    PA_FAIL(PA_ERR_INVALID, "bad block mask geometry");
+  if ((int64_t)kv_lo + (int64_t)nK * kv_block > Skv)
+    PA_FAIL(PA_ERR_INVALID, "key blocks [%d + %d*%d) exceed Skv=%d", kv_lo, nK, kv_block, Skv);
+  if (runs_ws_bytes < pa_blocksparse_workspace_bytes(Hm, nQ, nK))
+    PA_FAIL(PA_ERR_WORKSPACE, "runs workspace too small");
+  const int total = Hm * (nQ + 2);
+  const int cap = nK / 2 + 3;
+  hipLaunchKernelGGL(build_runs_kernel, dim3((total + 63) / 64), dim3(64), 0, (hipStream_t)stream,
+                     block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, cap, runs_ws);
+  PA_CHECK_LAUNCH("build_runs_kernel");
+  return PA_OK;
+}
+
+extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void* v, void* out,
+                                       float* lse, int dtype, int B, int H, int Sq, int Skv, int D,
+                                       const int64_t q_strides[3], const int64_t k_strides[3],
+                                       const int64_t v_strides[3], const int64_t out_strides[3],
+                                       float scale, const uint8_t* block_mask, int Hm, int nQ, int nK,
+                                       int q_lo, int q_block, int kv_lo, int kv_block,
+                                       int32_t* runs_ws, size_t runs_ws_bytes, void* stream) {
+  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                        out_strides, scale);
+  if (rc) return rc;
+  if (Hm != 1 && Hm != H) PA_FAIL(PA_ERR_INVALID, "block mask heads must be 1 or H=%d (got %d)", H, Hm);
+  if (q_block <= 0 || q_lo < 0 || (int64_t)q_lo + (int64_t)nQ * q_block > Sq)
+    PA_FAIL(PA_ERR_INVALID, "query blocks [%d + %d*%d) exceed Sq=%d", q_lo, nQ, q_block, Sq);
+  rc = pa_blocksparse_build_runs(block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, runs_ws, runs_ws_bytes, stream);
+  if (rc) return rc;
+  AttnParams p;
+  fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
+  p.runs = runs_ws;
+  p.Hm = Hm; p.nQ = nQ; p.cap = nK / 2 + 3;
+  p.q_lo = q_lo; p.q_block = q_block;
+  p.tiles_left = (q_lo + BM - 1) / BM;
+  p.tiles_per_block = (q_block + BM - 1) / BM;
+  const int q_hi = q_lo + nQ * q_block;
+  const int tiles_right = (Sq - q_hi + BM - 1) / BM;
+  p.n_qtiles = p.tiles_left + nQ * p.tiles_per_block + tiles_right;
+  return dispatch_attn<true>(p, dtype, D, (hipStream_t)stream);
+}

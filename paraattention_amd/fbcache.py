@@ -1,0 +1,189 @@
+"""First Block Cache decision path with the reference's function names
+(src/para_attn/first_block_cache/utils.py:12-120, 193-295): the cache context,
+the gates of ``get_can_use_cache`` and ``are_two_tensors_similar``, whose
+seven-launch reduction is one kernel here.  Only what the decision needs is
+kept; TaylorSeer, the diffusers adapters and the block orchestration are not
+part of this package.
+"""
+import contextlib
+import dataclasses
+from typing import Any, Dict, Optional, Union
+
+import torch
+
+from . import ops
+
+
+@dataclasses.dataclass
+class CacheContext:
+    """State of one pipeline call (reference fields of the same names, utils.py:12-37)."""
+
+    residual_diff_threshold: Union[torch.Tensor, float] = 0.0
+    alter_residual_diff_threshold: Optional[Union[torch.Tensor, float]] = None
+    downsample_factor: int = 1
+    enable_alter_cache: bool = False
+    num_inference_steps: int = -1
+    warmup_steps: int = 0
+    buffers: Dict[str, Any] = dataclasses.field(default_factory=dict)
+    executed_steps: int = 0
+    is_alter_cache: bool = True
+
+    def get_residual_diff_threshold(self):
+        if self.enable_alter_cache and self.is_alter_cache and self.alter_residual_diff_threshold is not None:
+            thr = self.alter_residual_diff_threshold
+        else:
+            thr = self.residual_diff_threshold
+        if isinstance(thr, torch.Tensor):
+            thr = thr.item()
+        return thr
+
+    def _name(self, name):
+        return f"{name}_alter" if self.enable_alter_cache and self.is_alter_cache else name
+
+    def get_buffer(self, name):
+        return self.buffers.get(self._name(name))
+
+    def set_buffer(self, name, buffer):
+        self.buffers[self._name(name)] = buffer
+
+    def remove_buffer(self, name):
+        self.buffers.pop(self._name(name), None)
+
+    def clear_buffers(self):
+        self.buffers.clear()
+
+    def mark_step_begin(self):
+        if not self.enable_alter_cache:
+            self.executed_steps += 1
+        else:
+            self.is_alter_cache = not self.is_alter_cache
+            if not self.is_alter_cache:
+                self.executed_steps += 1
+
+    def get_current_step(self):
+        return self.executed_steps - 1
+
+    def is_in_warmup(self):
+        return self.get_current_step() < self.warmup_steps
+
+
+_current_cache_context = None
+
+
+def create_cache_context(*args, **kwargs):
+    return CacheContext(*args, **kwargs)
+
+
+def get_current_cache_context():
+    return _current_cache_context
+
+
+def set_current_cache_context(cache_context=None):
+    global _current_cache_context
+    _current_cache_context = cache_context
+
+
+@contextlib.contextmanager
+def cache_context(cache_context):
+    global _current_cache_context
+    old = _current_cache_context
+    _current_cache_context = cache_context
+    try:
+        yield
+    finally:
+        _current_cache_context = old
+
+
+def _ctx():
+    ctx = get_current_cache_context()
+    assert ctx is not None, "cache_context must be set before"
+    return ctx
+
+
+def residual_diff(t1, t2):
+    """The 0-d ratio tensor ``mean|t1 - t2| / mean|t1|`` of utils.py:228-233, one kernel."""
+    return ops.fbcache_residual_diff(t1, t2)
+
+
+@torch.compiler.disable
+def are_two_tensors_similar(t1, t2, *, threshold, parallelized=False):
+    """utils.py:220-234.  ``parallelized`` would average the two means over ranks;
+    this build runs on one GPU and refuses it."""
+    if threshold <= 0.0:
+        return False
+    if t1.shape != t2.shape:
+        return False
+    if parallelized:
+        raise NotImplementedError("cross-rank averaging of the means needs more than one GPU")
+    diff = residual_diff(t1, t2)
+    return diff.item() < threshold
+
+
+@torch.compiler.disable
+def get_first_hidden_states_residual():
+    return _ctx().get_buffer("first_hidden_states_residual")
+
+
+@torch.compiler.disable
+def set_first_hidden_states_residual(first_hidden_states_residual):
+    """utils.py:289-295: the stored copy is the down-sampled, contiguous one."""
+    k = _ctx().downsample_factor
+    if k > 1:
+        first_hidden_states_residual = first_hidden_states_residual[..., ::k].contiguous()
+    _ctx().set_buffer("first_hidden_states_residual", first_hidden_states_residual)
+
+
+@torch.compiler.disable
+def get_can_use_cache(first_hidden_states_residual, parallelized=False):
+    """utils.py:269-286: warm-up gate, threshold gate, down-sampling, missing-previous gate, then the reduction."""
+    ctx = _ctx()
+    if ctx.is_in_warmup():
+        return False
+    threshold = ctx.get_residual_diff_threshold()
+    if threshold <= 0.0:
+        return False
+    k = ctx.downsample_factor
+    if k > 1:
+        first_hidden_states_residual = first_hidden_states_residual[..., ::k]
+    prev = get_first_hidden_states_residual()
+    return prev is not None and are_two_tensors_similar(
+        prev, first_hidden_states_residual, threshold=threshold, parallelized=parallelized
+    )
+
+
+@torch.compiler.disable
+def first_block_step(hidden_states, original_hidden_states, parallelized=False):
+    """Residual of the first block plus the cache decision in one pass over memory
+    (utils.py:359-366: ``hidden - original``, ``mark_step_begin``, ``get_can_use_cache``).
+
+    Returns (first_hidden_states_residual, can_use_cache).  Falls back to the
+    two-step form when down-sampling is on, since the stored residual then has
+    another shape than the fresh one.
+    """
+    ctx = _ctx()
+    ctx.mark_step_begin()
+    threshold = ctx.get_residual_diff_threshold()
+    gated = ctx.is_in_warmup() or threshold <= 0.0
+    prev = None if gated else get_first_hidden_states_residual()
+    if ctx.downsample_factor > 1 or (prev is not None and prev.shape != hidden_states.shape):
+        resid, _ = ops.fbcache_first_residual_diff(hidden_states, original_hidden_states, None)
+        return resid, (not gated) and get_can_use_cache(resid, parallelized=parallelized)
+    if parallelized and prev is not None:
+        raise NotImplementedError("cross-rank averaging of the means needs more than one GPU")
+    resid, ratio = ops.fbcache_first_residual_diff(hidden_states, original_hidden_states, prev)
+    can_use = prev is not None and ratio.item() < threshold
+    return resid, can_use
+
+
+@torch.compiler.disable
+def apply_prev_hidden_states_residual(hidden_states, encoder_hidden_states=None):
+    """Cache hit (utils.py:237-259): add the stored residuals back."""
+    ctx = _ctx()
+    res = ctx.get_buffer("hidden_states_residual")
+    assert res is not None, "hidden_states_residual must be set before"
+    hidden_states = ops.fbcache_apply_residual(res, hidden_states)
+    if encoder_hidden_states is not None:
+        eres = ctx.get_buffer("encoder_hidden_states_residual")
+        assert eres is not None, "encoder_hidden_states_residual must be set before"
+        encoder_hidden_states = ops.fbcache_apply_residual(eres, encoder_hidden_states)
+    return hidden_states, encoder_hidden_states

@@ -1,0 +1,524 @@
+"""The attention op layer: same op names and schemas as the reference's
+``para_attn.ops`` (src/para_attn/ops/__init__.py:160-343), backed by the gfx950
+kernels of libparaattn_hip.so instead of aten CUDA kernels.
+
+Registered in the ``para_attn`` namespace so ``torch.ops.para_attn.<name>`` and
+``torch.compile`` graphs resolve exactly as they do with the reference.  The ops
+exist for device type "cuda" only (which is what ROCm devices report): a CPU
+tensor raises from the dispatcher, as the reference's own assert does
+(src/para_attn/ops/__init__.py:123).
+
+Ops with a counterpart in the reference:
+  attention_forward_with_lse   (ops/__init__.py:160-201)
+  attention_forward            (ops/__init__.py:204-245)
+  attention_forward_sparse_kv  (ops/__init__.py:248-343)
+Ops the reference has no name for, because there the arithmetic is a chain of
+torch elementwise calls:
+  merge_attention_lse / merge_attention_lse_   (torch _SDPAMerger._merge_one)
+  attention_forward_block_sparse               (sparse_attn.py:74-278)
+  fbcache_residual_diff                        (first_block_cache/utils.py:228-233)
+  fbcache_first_residual_diff, fbcache_apply_residual (utils.py:359, 237-259)
+"""
+import ctypes
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.bfloat16: _lib.PA_DTYPE_BF16, torch.float16: _lib.PA_DTYPE_F16, torch.float32: _lib.PA_DTYPE_F32}
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _kernel_ready(t):
+    """Rows must be unit-stride and 16-byte aligned for the kernels' vector loads."""
+    if t.stride(-1) != 1 or any(t.shape[d] > 1 and t.stride(d) % 8 for d in range(t.ndim - 1)) or t.data_ptr() % 16:
+        return t.contiguous()
+    return t
+
+
+def _check_sdpa_args(query, key, value, dropout_p, is_causal):
+    if query.ndim != 4 or key.ndim != 4 or value.ndim != 4:
+        raise ValueError("query, key and value must be 4-D [batch, heads, seq, head_dim]")
+    if dropout_p != 0.0:
+        raise NotImplementedError("dropout_p > 0 is not supported (the reference's hot path is inference only)")
+    if is_causal:
+        raise NotImplementedError("is_causal=True is not supported by the gfx950 attention kernel")
+    if query.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError(f"attention dtype {query.dtype} not supported (bf16 / fp16)")
+    if key.dtype != query.dtype or value.dtype != query.dtype:
+        raise ValueError("query, key and value must share one dtype")
+    B, H, Sq, D = query.shape
+    if key.shape[0] != B or key.shape[1] != H or key.shape[3] != D:
+        raise ValueError(f"key shape {tuple(key.shape)} does not match query {tuple(query.shape)}")
+    if value.shape[:3] != key.shape[:3] or value.shape[3] != D:
+        raise ValueError(f"value shape {tuple(value.shape)} does not match key {tuple(key.shape)}")
+
+
+def _key_keep_vector(attn_mask, B, Skv):
+    """Reduce a boolean mask that only selects keys to [B, Skv], or return None.
+
+    Accepts the shapes the reference's sparse_kv op accepts (any leading dims,
+    reduced to their first head / first query row, src/para_attn/ops/__init__.py:280-282).
+    """
+    m = attn_mask
+    if m.dtype != torch.bool or m.shape[-1] != Skv:
+        return None
+    while m.ndim > 2:
+        if m.shape[1] != 1:
+            return None
+        m = m[:, 0]
+    if m.ndim == 1:
+        m = m.unsqueeze(0)
+    if m.shape[0] not in (1, B):
+        return None
+    return m.expand(B, Skv)
+
+
+def _dense_forward(query, key, value, scale, want_lse, kv_len=None):
+    B, H, Sq, D = query.shape
+    Skv = key.shape[2]
+    q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
+    out = torch.empty_like(q)
+    if out.stride(-1) != 1:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        rc = lib.pa_attn_fwd_lse(
+            _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
+            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+            float(scale), _ptr(kv_len), _stream_ptr(q.device),
+        )
+    _lib.check(rc, "pa_attn_fwd_lse")
+    return out, lse
+
+
+def _masked_forward(query, key, value, attn_mask, scale, want_lse):
+    """attn_mask handling shared by the three SDPA-signature ops."""
+    if attn_mask is None:
+        return _dense_forward(query, key, value, scale, want_lse)
+    B, Skv = query.shape[0], key.shape[2]
+    keep = _key_keep_vector(attn_mask, B, Skv)
+    if keep is None:
+        raise NotImplementedError(
+            "attn_mask must be None or a boolean mask over keys only ([B,1,1,Skv]-like); "
+            "per-query masks go through attention_forward_block_sparse"
+        )
+    lens = keep.sum(-1, dtype=torch.int32)
+    prefix = torch.arange(Skv, device=keep.device).unsqueeze(0) < lens.unsqueeze(1)
+    if not bool((keep == prefix).all()):
+        # kept keys are scattered: move them to the front (stable), then treat as a prefix
+        order = torch.argsort((~keep).to(torch.uint8), dim=-1, stable=True)
+        idx = order[:, None, :, None].expand(B, key.shape[1], Skv, key.shape[3])
+        key = torch.gather(key, 2, idx)
+        value = torch.gather(value, 2, idx)
+    return _dense_forward(query, key, value, scale, want_lse, kv_len=lens.contiguous())
+
+
+# ---------------------------------------------------------------------------------
+# ops that exist in the reference
+# ---------------------------------------------------------------------------------
+@torch.library.custom_op("para_attn::attention_forward_with_lse", mutates_args=(), device_types=("cuda",))
+def attention_forward_with_lse(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    dropout_p: float = 0.0,
+    is_causal: bool = False,
+    *,
+    scale: Optional[float] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """out [B,H,Sq,D] in query's dtype and natural-log LSE [B,H,Sq] in fp32
+    (src/para_attn/ops/__init__.py:160-179)."""
+    _check_sdpa_args(query, key, value, dropout_p, is_causal)
+    out, lse = _masked_forward(query, key, value, attn_mask, scale, True)
+    return out, lse
+
+
+@torch.library.register_fake("para_attn::attention_forward_with_lse")
+def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
+    B, H, Sq, _ = query.shape
+    out = query.new_empty((B, H, Sq, value.shape[-1]))
+    lse = query.new_empty((B, H, Sq), dtype=torch.float32)
+    return out, lse
+
+
+@torch.library.custom_op("para_attn::attention_forward", mutates_args=(), device_types=("cuda",))
+def attention_forward(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    dropout_p: float = 0.0,
+    is_causal: bool = False,
+    *,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Plain SDPA forward, no LSE (src/para_attn/ops/__init__.py:204-223)."""
+    _check_sdpa_args(query, key, value, dropout_p, is_causal)
+    out, _ = _masked_forward(query, key, value, attn_mask, scale, False)
+    return out
+
+
+@torch.library.register_fake("para_attn::attention_forward")
+def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
+    B, H, Sq, _ = query.shape
+    return query.new_empty((B, H, Sq, value.shape[-1]))
+
+
+@torch.library.custom_op("para_attn::attention_forward_sparse_kv", mutates_args=(), device_types=("cuda",))
+def attention_forward_sparse_kv(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    dropout_p: float = 0.0,
+    is_causal: bool = False,
+    *,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """SDPA over the keys a boolean mask keeps (src/para_attn/ops/__init__.py:248-321).
+
+    As in the reference the mask is reduced to its first head and first query
+    row per batch element (ops/__init__.py:280-282), must be boolean (:269) and
+    excludes is_causal (:270).  A prefix mask (valid text length) costs nothing:
+    the kernel just stops at the per-batch key count.
+    """
+    _check_sdpa_args(query, key, value, dropout_p, is_causal)
+    if attn_mask is None:
+        return _dense_forward(query, key, value, scale, False)[0]
+    if attn_mask.dtype != torch.bool:
+        raise AssertionError("attn_mask must be a boolean tensor")
+    m = attn_mask
+    if m.shape[0] != query.shape[0]:
+        m = m.expand(query.shape[0], *m.shape[1:])
+    while m.ndim > 2:
+        m = m[:, 0]
+    out, _ = _masked_forward(query, key, value, m[:, None, None, :], scale, False)
+    return out
+
+
+@torch.library.register_fake("para_attn::attention_forward_sparse_kv")
+def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
+    B, H, Sq, _ = query.shape
+    return query.new_empty((B, H, Sq, value.shape[-1]))
+
+
+# ---------------------------------------------------------------------------------
+# merge of partial attention results
+# ---------------------------------------------------------------------------------
+def _merge_launch(acc_out, acc_lse, blk_out, blk_lse, out, lse_out):
+    D = acc_out.shape[-1]
+    rows = acc_out.numel() // D if D else 0
+    lib = _lib.load()
+    with torch.cuda.device(acc_out.device):
+        rc = lib.pa_merge_lse(
+            _ptr(acc_out), _DTYPE_CODE[acc_out.dtype], _ptr(acc_lse),
+            _ptr(blk_out), _DTYPE_CODE[blk_out.dtype], _ptr(blk_lse),
+            _ptr(out), _DTYPE_CODE[out.dtype], _ptr(lse_out), rows, D, _stream_ptr(acc_out.device),
+        )
+    _lib.check(rc, "pa_merge_lse")
+
+
+def _check_merge_args(acc_out, acc_lse, blk_out, blk_lse):
+    if acc_out.shape != blk_out.shape:
+        raise ValueError(f"partial outputs differ in shape: {tuple(acc_out.shape)} vs {tuple(blk_out.shape)}")
+    rows = acc_out.numel() // max(acc_out.shape[-1], 1)
+    if acc_lse.numel() != rows or blk_lse.numel() != rows:
+        raise ValueError("LSE must have one value per output row ([...,Sq] or [...,Sq,1])")
+    if acc_lse.dtype != torch.float32 or blk_lse.dtype != torch.float32:
+        raise NotImplementedError("LSE must be fp32")
+    for t in (acc_out, blk_out):
+        if t.dtype not in _DTYPE_CODE:
+            raise NotImplementedError(f"dtype {t.dtype} not supported by the merge kernel")
+
+
+@torch.library.custom_op("para_attn::merge_attention_lse", mutates_args=(), device_types=("cuda",))
+def merge_attention_lse(
+    acc_out: torch.Tensor,
+    acc_lse: torch.Tensor,
+    blk_out: torch.Tensor,
+    blk_lse: torch.Tensor,
+    out_dtype: Optional[torch.dtype] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One functional merge step: returns (out, lse) of the two partial results combined.
+
+    out = acc_out - sigmoid(blk_lse - acc_lse) * (acc_out - blk_out)
+    lse = acc_lse - logsigmoid(acc_lse - blk_lse)
+    (torch _SDPAMerger._merge_one, _context_parallel/_attention.py:182-183), in
+    fp32.  ``out_dtype`` defaults to fp32 (the merger's convert_to_f32 mode);
+    pass the activation dtype on the last step to fold results()'s cast.
+    The returned lse has acc_lse's shape.
+    """
+    _check_merge_args(acc_out, acc_lse, blk_out, blk_lse)
+    a, b = acc_out.contiguous(), blk_out.contiguous()
+    la, lb = acc_lse.contiguous(), blk_lse.contiguous()
+    out = torch.empty(a.shape, dtype=out_dtype or torch.float32, device=a.device)
+    lse = torch.empty(la.shape, dtype=torch.float32, device=a.device)
+    _merge_launch(a, la, b, lb, out, lse)
+    return out, lse
+
+
+@torch.library.register_fake("para_attn::merge_attention_lse")
+def _(acc_out, acc_lse, blk_out, blk_lse, out_dtype=None):
+    return (
+        acc_out.new_empty(acc_out.shape, dtype=out_dtype or torch.float32),
+        acc_lse.new_empty(acc_lse.shape, dtype=torch.float32),
+    )
+
+
+@torch.library.custom_op("para_attn::merge_attention_lse_", mutates_args=("acc_out", "acc_lse"), device_types=("cuda",))
+def merge_attention_lse_(
+    acc_out: torch.Tensor, acc_lse: torch.Tensor, blk_out: torch.Tensor, blk_lse: torch.Tensor
+) -> None:
+    """In-place merge step: folds (blk_out, blk_lse) into the contiguous accumulators."""
+    _check_merge_args(acc_out, acc_lse, blk_out, blk_lse)
+    if not acc_out.is_contiguous() or not acc_lse.is_contiguous():
+        raise ValueError("in-place merge needs contiguous accumulators")
+    _merge_launch(acc_out, acc_lse, blk_out.contiguous(), blk_lse.contiguous(), acc_out, acc_lse)
+
+
+@torch.library.register_fake("para_attn::merge_attention_lse_")
+def _(acc_out, acc_lse, blk_out, blk_lse):
+    return None
+
+
+# ---------------------------------------------------------------------------------
+# block-sparse attention
+# ---------------------------------------------------------------------------------
+@torch.library.custom_op("para_attn::attention_forward_block_sparse", mutates_args=(), device_types=("cuda",))
+def attention_forward_block_sparse(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    block_mask: torch.Tensor,
+    q_lo: int = 0,
+    q_hi: int = -1,
+    kv_lo: int = 0,
+    kv_hi: int = -1,
+    *,
+    scale: Optional[float] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Attention restricted to the kept tiles of ``block_mask``; returns (out, fp32 LSE).
+
+    block_mask: bool [nQ,nK] (shared by batch and heads, the reference's form,
+    src/para_attn/sparse_attn.py:107) or [H,nQ,nK].  Query rows [q_lo,q_hi) are
+    cut into nQ equal blocks and keys [kv_lo,kv_hi) into nK equal blocks
+    (sparse_range_query / sparse_range_key_value, sparse_attn.py:112-131);
+    rows and keys outside those ranges are dense (:158-171, :178-189, :247-274).
+    Identical to dense SDPA with -inf on the dropped tiles.
+    """
+    _check_sdpa_args(query, key, value, 0.0, False)
+    B, H, Sq, D = query.shape
+    Skv = key.shape[2]
+    q_hi = Sq if q_hi < 0 else q_hi
+    kv_hi = Skv if kv_hi < 0 else kv_hi
+    if block_mask.dtype != torch.bool:
+        raise ValueError("block_mask must be boolean")
+    if block_mask.ndim == 2:
+        block_mask = block_mask.unsqueeze(0)
+    if block_mask.ndim != 3 or block_mask.shape[0] not in (1, H):
+        raise ValueError(f"block_mask must be [nQ,nK] or [H,nQ,nK], got {tuple(block_mask.shape)}")
+    Hm, nQ, nK = block_mask.shape
+    if not (0 <= q_lo <= q_hi <= Sq):
+        raise ValueError(f"sparse query range must be in [0, {Sq}], got {(q_lo, q_hi)}")
+    if not (0 <= kv_lo <= kv_hi <= Skv):
+        raise ValueError(f"sparse key/value range must be in [0, {Skv}], got {(kv_lo, kv_hi)}")
+    if nQ == 0 or nK == 0 or (q_hi - q_lo) % nQ or (kv_hi - kv_lo) % nK:
+        raise ValueError("block_mask must divide the sparse query and key/value ranges")
+    q_block = (q_hi - q_lo) // nQ
+    kv_block = (kv_hi - kv_lo) // nK
+    if q_block == 0 or kv_block == 0:
+        raise ValueError("empty sparse range")
+    q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
+    out = torch.empty_like(q)
+    if out.stride(-1) != 1:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    mask_u8 = block_mask.contiguous().view(torch.uint8)
+    lib = _lib.load()
+    ws_bytes = lib.pa_blocksparse_workspace_bytes(Hm, nQ, nK)
+    ws = torch.empty((ws_bytes + 3) // 4, dtype=torch.int32, device=q.device)
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    with torch.cuda.device(q.device):
+        rc = lib.pa_attn_fwd_blocksparse(
+            _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
+            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out), float(scale),
+            _ptr(mask_u8), Hm, nQ, nK, q_lo, q_block, kv_lo, kv_block, _ptr(ws), ws_bytes,
+            _stream_ptr(q.device),
+        )
+    _lib.check(rc, "pa_attn_fwd_blocksparse")
+    return out, lse
+
+
+@torch.library.register_fake("para_attn::attention_forward_block_sparse")
+def _(query, key, value, block_mask, q_lo=0, q_hi=-1, kv_lo=0, kv_hi=-1, *, scale=None):
+    B, H, Sq, _ = query.shape
+    return query.new_empty((B, H, Sq, value.shape[-1])), query.new_empty((B, H, Sq), dtype=torch.float32)
+
+
+def block_sparse_runs(block_mask, Skv, kv_lo=0, kv_hi=-1):
+    """Key ranges the block-sparse kernel walks, per (mask head, query segment), as the device built them.
+
+    Returns (count [Hm, nQ+2] int32, ranges [Hm, nQ+2, cap, 2] int32) on the mask's device.
+    """
+    if block_mask.ndim == 2:
+        block_mask = block_mask.unsqueeze(0)
+    Hm, nQ, nK = block_mask.shape
+    kv_hi = Skv if kv_hi < 0 else kv_hi
+    kv_block = (kv_hi - kv_lo) // nK
+    lib = _lib.load()
+    ws_bytes = lib.pa_blocksparse_workspace_bytes(Hm, nQ, nK)
+    ws = torch.zeros((ws_bytes + 3) // 4, dtype=torch.int32, device=block_mask.device)
+    mask_u8 = block_mask.contiguous().view(torch.uint8)
+    with torch.cuda.device(block_mask.device):
+        rc = lib.pa_blocksparse_build_runs(
+            _ptr(mask_u8), Hm, nQ, nK, Skv, kv_lo, kv_block, _ptr(ws), ws_bytes, _stream_ptr(block_mask.device)
+        )
+    _lib.check(rc, "pa_blocksparse_build_runs")
+    nseg, cap = nQ + 2, nK // 2 + 3
+    count = ws[: Hm * nseg].view(Hm, nseg)
+    ranges = ws[Hm * nseg : Hm * nseg + Hm * nseg * cap * 2].view(Hm, nseg, cap, 2)
+    return count, ranges
+
+
+# ---------------------------------------------------------------------------------
+# First Block Cache reductions
+# ---------------------------------------------------------------------------------
+_fb_workspaces = {}
+
+
+def _fb_workspace(device):
+    """Zero-initialised ticket/partials buffer, one per (device, stream)."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _fb_workspaces.get(key)
+    if ws is None:
+        nbytes = _lib.load().pa_fbcache_workspace_bytes()
+        ws = torch.zeros((nbytes + 7) // 8, dtype=torch.int64, device=device)
+        _fb_workspaces[key] = ws
+    return ws
+
+
+def _as_rows(t):
+    """View a tensor as [rows, row_len] with (row_stride, col_stride) without copying, or None."""
+    if t.ndim == 0:
+        return 1, 1, 1, 1
+    row_len = t.shape[-1]
+    col_stride = t.stride(-1) if row_len > 1 else 1
+    lead = t.shape[:-1]
+    rows = 1
+    for s in lead:
+        rows *= s
+    if rows <= 1:
+        return max(rows, 0), row_len, row_len * col_stride, col_stride
+    # leading dims must collapse to one stride
+    expect = None
+    for d in range(t.ndim - 2, -1, -1):
+        if t.shape[d] == 1:
+            continue
+        if expect is None:
+            row_stride = t.stride(d)
+            expect = t.stride(d) * t.shape[d]
+        else:
+            if t.stride(d) != expect:
+                return None
+            expect = t.stride(d) * t.shape[d]
+    return rows, row_len, row_stride, col_stride
+
+
+@torch.library.custom_op("para_attn::fbcache_residual_diff", mutates_args=(), device_types=("cuda",))
+def fbcache_residual_diff(prev: torch.Tensor, cur: torch.Tensor) -> torch.Tensor:
+    """0-d tensor ``(prev - cur).abs().mean() / prev.abs().mean()`` in the activation dtype,
+    with torch's rounding of every intermediate (src/para_attn/first_block_cache/utils.py:228-233).
+    ``cur`` may be a strided view such as ``x[..., ::k]`` (utils.py:276-278)."""
+    if prev.shape != cur.shape:
+        raise ValueError(f"shape mismatch {tuple(prev.shape)} vs {tuple(cur.shape)}")
+    if prev.dtype != cur.dtype or prev.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"dtypes {prev.dtype}/{cur.dtype} not supported")
+    if prev.numel() == 0:
+        raise ValueError("mean of an empty tensor")
+    pr, cr = _as_rows(prev), _as_rows(cur)
+    if pr is None:
+        prev = prev.contiguous()
+        pr = _as_rows(prev)
+    if cr is None:
+        cur = cur.contiguous()
+        cr = _as_rows(cur)
+    ratio = torch.empty((), dtype=prev.dtype, device=prev.device)
+    ws = _fb_workspace(prev.device)
+    lib = _lib.load()
+    with torch.cuda.device(prev.device):
+        rc = lib.pa_fbcache_absdiff_ratio(
+            _ptr(prev), _ptr(cur), _DTYPE_CODE[prev.dtype], pr[0], pr[1], pr[2], pr[3], cr[2], cr[3],
+            _ptr(ratio), None, _ptr(ws), ws.numel() * 8, _stream_ptr(prev.device),
+        )
+    _lib.check(rc, "pa_fbcache_absdiff_ratio")
+    return ratio
+
+
+@torch.library.register_fake("para_attn::fbcache_residual_diff")
+def _(prev, cur):
+    return prev.new_empty(())
+
+
+@torch.library.custom_op("para_attn::fbcache_first_residual_diff", mutates_args=(), device_types=("cuda",))
+def fbcache_first_residual_diff(
+    hidden: torch.Tensor, hidden0: torch.Tensor, prev: Optional[torch.Tensor] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(residual, ratio): residual = hidden - hidden0 (src/para_attn/first_block_cache/utils.py:359)
+    and, in the same pass, the reduction of ``fbcache_residual_diff(prev, residual)``.
+    Without ``prev`` the ratio is +inf (never similar)."""
+    if hidden.shape != hidden0.shape or hidden.dtype != hidden0.dtype or hidden.dtype not in _DTYPE_CODE:
+        raise ValueError("hidden and hidden0 must share shape and a supported dtype")
+    if prev is not None and (prev.shape != hidden.shape or prev.dtype != hidden.dtype):
+        raise ValueError("prev must match hidden in shape and dtype")
+    h, h0 = hidden.contiguous(), hidden0.contiguous()
+    pv = prev.contiguous() if prev is not None else None
+    resid = torch.empty(h.shape, dtype=h.dtype, device=h.device)
+    ratio = torch.full((), float("inf"), dtype=h.dtype, device=h.device)
+    ws = _fb_workspace(h.device)
+    lib = _lib.load()
+    with torch.cuda.device(h.device):
+        rc = lib.pa_fbcache_residual_ratio(
+            _ptr(h), _ptr(h0), _ptr(pv), _ptr(resid), _DTYPE_CODE[h.dtype], h.numel(), _ptr(ratio), None,
+            _ptr(ws), ws.numel() * 8, _stream_ptr(h.device),
+        )
+    _lib.check(rc, "pa_fbcache_residual_ratio")
+    return resid, ratio
+
+
+@torch.library.register_fake("para_attn::fbcache_first_residual_diff")
+def _(hidden, hidden0, prev=None):
+    return hidden.new_empty(hidden.shape), hidden.new_empty(())
+
+
+@torch.library.custom_op("para_attn::fbcache_apply_residual", mutates_args=(), device_types=("cuda",))
+def fbcache_apply_residual(residual: torch.Tensor, hidden: torch.Tensor) -> torch.Tensor:
+    """``residual + hidden``, contiguous (src/para_attn/first_block_cache/utils.py:237-259)."""
+    if residual.shape != hidden.shape or residual.dtype != hidden.dtype or hidden.dtype not in _DTYPE_CODE:
+        raise ValueError("residual and hidden must share shape and a supported dtype")
+    r, h = residual.contiguous(), hidden.contiguous()
+    out = torch.empty(h.shape, dtype=h.dtype, device=h.device)
+    lib = _lib.load()
+    with torch.cuda.device(h.device):
+        rc = lib.pa_fbcache_apply_residual(_ptr(r), _ptr(h), _ptr(out), _DTYPE_CODE[h.dtype], h.numel(), _stream_ptr(h.device))
+    _lib.check(rc, "pa_fbcache_apply_residual")
+    return out
+
+
+@torch.library.register_fake("para_attn::fbcache_apply_residual")
+def _(residual, hidden):
+    return hidden.new_empty(hidden.shape)

@@ -1,0 +1,170 @@
+"""Parity of the HIP attention kernel (through torch.ops.para_attn.* -> C ABI) with the oracle.
+
+Tolerances are the ones the task states: bf16/fp16 output atol 2e-2 / rtol 2e-2, fp32 LSE 1e-3.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import paraattention_amd  # noqa: F401
+from oracle import attention as oattn
+from oracle import inputs
+
+pytestmark = pytest.mark.gpu
+
+OUT_ATOL = OUT_RTOL = 2e-2
+LSE_ATOL = 1e-3
+
+
+def _check(out, lse, ref_out, ref_lse, what=""):
+    out = out.float().cpu().numpy().astype(np.float64)
+    ref_out = np.asarray(ref_out, dtype=np.float64)
+    err = np.abs(out - ref_out)
+    tol = OUT_ATOL + OUT_RTOL * np.abs(ref_out)
+    assert (err <= tol).all(), f"{what}: out max err {err.max():.4g} (worst excess {(err - tol).max():.4g})"
+    if lse is not None:
+        lse = lse.cpu().numpy().astype(np.float64)
+        lerr = np.abs(lse - np.asarray(ref_lse, dtype=np.float64))
+        assert lse.dtype == np.float64 and (lerr <= LSE_ATOL).all(), f"{what}: lse max err {lerr.max():.4g}"
+
+
+# ragged sizes the reference's shapes hit: 119056 = 930*128 + 16, 14882 = 116*128 + 34, 32760 = 255*128 + 120
+SMALL = [
+    (1, 1, 1, 1), (1, 2, 15, 17), (2, 3, 16, 16), (1, 2, 17, 34), (1, 1, 33, 63), (1, 2, 64, 64), (1, 1, 65, 65),
+    (1, 2, 120, 129), (1, 1, 128, 128), (1, 3, 129, 120), (2, 2, 257, 300), (1, 2, 300, 1000), (1, 1, 1000, 77),
+]
+
+
+@pytest.mark.parametrize("B,H,Sq,Skv", SMALL)
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_vs_f64(cuda, B, H, Sq, Skv, D, dtype):
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=Sq * 1000 + Skv, dtype=dtype)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
+    assert out.dtype == dtype and out.shape == (B, H, Sq, D)
+    assert lse.dtype == torch.float32 and lse.shape == (B, H, Sq)  # the reference's own assertions, tests/ops/test_ops.py:63-64
+    _check(out, lse, ref_out, ref_lse, f"{(B, H, Sq, Skv, D, dtype)}")
+    out2 = torch.ops.para_attn.attention_forward(q.to(cuda), k.to(cuda), v.to(cuda))
+    assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("scale", [0.05, 1.0, None])
+def test_scale_and_large_logits(cuda, scale):
+    # scaled logits up to a few hundred: exercises the running-maximum update
+    q, k, v = inputs.qkv(1, 2, 200, 500, 128, seed=7)
+    q = q * 4
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), scale=scale)
+    _check(out, lse, ref_out, ref_lse)
+
+
+def test_increasing_maximum(cuda):
+    # keys ordered so that every tile raises the row maximum: the rescale path runs on each tile
+    D, Skv = 128, 640
+    g = torch.Generator().manual_seed(3)
+    q = torch.ones(1, 1, 64, D) * 0.5
+    k = torch.randn(1, 1, Skv, D, generator=g) * 0.1 + torch.linspace(-2, 2, Skv)[None, None, :, None]
+    v = torch.randn(1, 1, Skv, D, generator=g)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), 1.0)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), scale=1.0)
+    _check(out, lse, ref_out, ref_lse)
+
+
+def test_closed_forms(cuda):
+    D = 128
+    q, k, v = inputs.qkv(1, 2, 77, 333, D, seed=11)
+    # K = 0: uniform weights -> out = mean(V), lse = ln(Skv)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), torch.zeros_like(k).to(cuda), v.to(cuda))
+    assert torch.allclose(lse.cpu(), torch.full_like(lse.cpu(), math.log(333)), atol=1e-4)
+    assert torch.allclose(out.float().cpu(), v.float().mean(2, keepdim=True).expand(-1, -1, 77, -1), atol=2e-2, rtol=2e-2)
+    # V constant along keys: out = that constant, exactly representable
+    vc = torch.full_like(v, 0.75)
+    out, _ = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), vc.to(cuda))
+    assert torch.allclose(out.float().cpu(), vc.float()[:, :, :1].expand(-1, -1, 77, -1), atol=4e-3)
+
+
+def test_noncontiguous_layouts(cuda):
+    # diffusers hands SDPA [B,S,H,D] memory viewed as [B,H,S,D]
+    B, H, S, D = 2, 3, 200, 128
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=5)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    qt, kt, vt = (t.to(cuda).transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
+    assert not qt.is_contiguous()
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qt, kt, vt)
+    assert out.stride() == qt.stride()  # output keeps the query's memory layout
+    _check(out, lse, ref_out, ref_lse)
+    # sliced views (non-dense strides)
+    big = torch.randn(B, H, S + 8, D + 64, generator=torch.Generator().manual_seed(1)).bfloat16()
+    qs = big[:, :, 3 : 3 + S, :D]
+    ref_out, ref_lse = oattn.sdpa_lse_f64(qs.float().numpy(), k.float().numpy(), v.float().numpy())
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(big.to(cuda)[:, :, 3 : 3 + S, :D], k.to(cuda), v.to(cuda))
+    _check(out, lse, ref_out, ref_lse)
+
+
+def test_permutation_invariance(cuda):
+    q, k, v = inputs.qkv(1, 2, 130, 515, 128, seed=9)
+    perm = torch.randperm(515, generator=torch.Generator().manual_seed(0))
+    o1, l1 = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
+    o2, l2 = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k[:, :, perm].to(cuda), v[:, :, perm].to(cuda))
+    assert torch.allclose(l1, l2, atol=1e-4)
+    assert torch.allclose(o1.float(), o2.float(), atol=2e-2, rtol=2e-2)
+
+
+def test_flux_shape_vs_torch_cpu(cuda):
+    # BASELINE config 1: B1 H24 S4608 D128 against torch's CPU SDPA on identical bits
+    q, k, v = inputs.qkv(1, 24, 4608, 4608, 128, seed=0)
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q, k, v)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
+    _check(out, lse, ref_out.float().numpy(), ref_lse.numpy(), "flux")
+
+
+def test_hunyuan_shape_sampled_rows(cuda):
+    # BASELINE config 2 at full size on the GPU; the oracle checks sampled query rows of each head
+    B, H, S, D = 1, 3, 119056, 128
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=0, rms_norm_qk=True)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
+    rows = torch.cat([torch.arange(0, 40), torch.arange(S - 40, S), torch.randint(0, S, (176,), generator=torch.Generator().manual_seed(1))])
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, :, rows], k, v)
+    _check(out[:, :, rows.to(cuda)], lse[:, :, rows.to(cuda)], ref_out.float().numpy(), ref_lse.numpy(), "hunyuan")
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+
+
+def test_wan_cross_attention_shape(cuda):
+    # BASELINE config 4 cross-attention: 32760 queries x 512 text keys (reduced heads for the CPU check)
+    q, k, v = inputs.qkv(1, 4, 32760, 512, 128, seed=2)
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q, k, v)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
+    _check(out, lse, ref_out.float().numpy(), ref_lse.numpy(), "wan-cross")
+
+
+def test_key_mask_and_sparse_kv(cuda):
+    B, H, Sq, Skv, D = 2, 2, 150, 333, 128
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=21)
+    # prefix mask (valid text length per batch element) and a scattered mask
+    lens = [333, 201]
+    prefix = torch.arange(Skv)[None, :] < torch.tensor(lens)[:, None]
+    scattered = torch.rand(B, Skv, generator=torch.Generator().manual_seed(4)) < 0.6
+    for m in (prefix, scattered):
+        keep = m[:, None, None, :].numpy()
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, keep)
+        mask4 = m[:, None, None, :].expand(B, 1, Sq, Skv).to(cuda)
+        out = torch.ops.para_attn.attention_forward_sparse_kv(q.to(cuda), k.to(cuda), v.to(cuda), mask4)
+        _check(out, None, ref_out, None, "sparse_kv")
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), m[:, None, None, :].to(cuda))
+        _check(out, lse, ref_out, ref_lse, "key mask")
+
+
+def test_unsupported_raise(cuda):
+    q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 128))
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward_with_lse(q, k, v, is_causal=True)
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward_with_lse(q, k, v, dropout_p=0.1)
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward_with_lse(q[..., :32], k[..., :32], v[..., :32])
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward_with_lse(q.float(), k.float(), v.float())

@@ -1,0 +1,104 @@
+"""Parity of the fused merge kernel and the ring sweep with the oracle and with torch's own merger."""
+import numpy as np
+import pytest
+import torch
+
+import paraattention_amd
+from oracle import attention as oattn
+from oracle import inputs
+from oracle import merge as omerge
+
+pytestmark = pytest.mark.gpu
+
+
+def _partials(B, H, S, D, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    o1 = torch.randn(B, H, S, D, generator=g).to(dtype)
+    o2 = torch.randn(B, H, S, D, generator=g).to(dtype)
+    l1 = torch.randn(B, H, S, generator=g) * 3 + 5
+    l2 = torch.randn(B, H, S, generator=g) * 3 + 5
+    return o1, l1, o2, l2
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 8), (1, 2, 34, 128), (2, 3, 257, 64), (1, 24, 1000, 128)])
+@pytest.mark.parametrize("blk_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_merge_step_vs_oracle(cuda, shape, blk_dtype):
+    B, H, S, D = shape
+    o1, l1, o2, l2 = _partials(B, H, S, D, seed=S, dtype=blk_dtype)
+    ref_out, ref_lse = omerge.merge_step(o1.float().numpy(), l1.numpy(), o2.float().numpy(), l2.numpy())
+    # functional: 16-bit accumulator in (the first real step), fp32 out
+    out, lse = torch.ops.para_attn.merge_attention_lse(o1.to(cuda), l1.to(cuda), o2.to(cuda), l2.to(cuda))
+    assert out.dtype == torch.float32 and lse.dtype == torch.float32 and lse.shape == l1.shape
+    np.testing.assert_allclose(out.cpu().numpy(), ref_out, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(lse.cpu().numpy(), ref_lse, rtol=1e-6, atol=2e-6)
+    # in-place on fp32 accumulators
+    acc, acc_l = o1.float().to(cuda), l1.clone().to(cuda)
+    torch.ops.para_attn.merge_attention_lse_(acc, acc_l, o2.to(cuda), l2.to(cuda))
+    assert torch.equal(acc, out) and torch.equal(acc_l, lse)
+    # final step writes the activation dtype directly = fp32 result rounded once
+    if blk_dtype != torch.float32:
+        outb, _ = torch.ops.para_attn.merge_attention_lse(o1.float().to(cuda), l1.to(cuda), o2.to(cuda), l2.to(cuda), blk_dtype)
+        assert torch.equal(outb, out.to(blk_dtype))
+    # LSE given as [B,H,S,1] (the cuDNN layout torch's merger also accepts)
+    out4, lse4 = torch.ops.para_attn.merge_attention_lse(o1.to(cuda), l1[..., None].to(cuda), o2.to(cuda), l2[..., None].to(cuda))
+    assert lse4.shape == (B, H, S, 1) and torch.equal(out4, out)
+
+
+def test_merge_vs_torch_sdpa_merger(cuda):
+    from torch.distributed.tensor.experimental._context_parallel._attention import _SDPAMerger
+
+    B, H, S, D = 1, 4, 300, 128
+    g = torch.Generator().manual_seed(0)
+    outs = [torch.randn(B, H, S, D, generator=g).bfloat16() for _ in range(5)]
+    lses = [torch.randn(B, H, S, generator=g) * 4 for _ in range(5)]
+    ref = _SDPAMerger(True, 2)
+    mine = paraattention_amd.SDPAMerger(True, 2)
+    for o, l in zip(outs, lses):
+        ref.step(o, l, False)
+        mine.step(o.to(cuda), l.to(cuda), False)
+    ro, rl = ref.results()
+    mo, ml = mine.results()
+    assert mo.dtype == ro.dtype and ml.shape == rl.shape
+    torch.testing.assert_close(ml.cpu(), rl, rtol=1e-6, atol=1e-5)
+    torch.testing.assert_close(mo.float().cpu(), ro.float(), rtol=1.6e-2, atol=1e-5)  # one bf16 ulp after fp32 merge
+
+
+def test_merge_empty_partials(cuda):
+    # a partial that saw no key (lse = -inf) is the identity, on either side
+    o1, l1, o2, l2 = _partials(1, 1, 64, 128, seed=1)
+    ninf = torch.full_like(l2, float("-inf"))
+    out, lse = torch.ops.para_attn.merge_attention_lse(o1.to(cuda), l1.to(cuda), torch.zeros_like(o2).to(cuda), ninf.to(cuda))
+    assert torch.equal(out.cpu(), o1.float()) and torch.equal(lse.cpu(), l1)
+    out, lse = torch.ops.para_attn.merge_attention_lse(torch.zeros_like(o1).to(cuda), ninf.to(cuda), o2.to(cuda), l2.to(cuda))
+    assert torch.equal(out.cpu(), o2.float()) and torch.equal(lse.cpu(), l2)
+
+
+def test_ring_sweep_equals_full_attention(cuda):
+    # BASELINE config 3 in miniature, ragged like 14882 = 116*128 + 34: 8 blocks of 290 keys
+    B, H, Sq, D, nblk, blk = 1, 4, 290, 128, 8, 290
+    q, k, v = inputs.qkv(B, H, Sq, nblk * blk, D, seed=3)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    kb = [k[:, :, i * blk : (i + 1) * blk].contiguous().to(cuda) for i in range(nblk)]
+    vb = [v[:, :, i * blk : (i + 1) * blk].contiguous().to(cuda) for i in range(nblk)]
+    out, lse = paraattention_amd.ring_sweep(q.to(cuda), kb, vb)
+    assert out.dtype == torch.bfloat16
+    np.testing.assert_allclose(lse.cpu().numpy(), ref_lse, atol=1e-3)
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+
+
+def test_ring_sweep_full_shape_sampled(cuda):
+    # BASELINE config 3 at full size (Q block 14882 x 24 heads against 8 KV blocks of 14882);
+    # the oracle checks sampled rows of two heads against one full-length SDPA over 119056 keys
+    B, H, Sq, D, nblk = 1, 24, 14882, 128, 8
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, H, Sq, D, generator=g).bfloat16()
+    kb_cpu = [torch.randn(B, H, Sq, D, generator=g).bfloat16() for _ in range(nblk)]
+    vb_cpu = [torch.randn(B, H, Sq, D, generator=g).bfloat16() for _ in range(nblk)]
+    out, lse = paraattention_amd.ring_sweep(q.to(cuda), [t.to(cuda) for t in kb_cpu], [t.to(cuda) for t in vb_cpu])
+    rows = torch.cat([torch.arange(0, 16), torch.arange(Sq - 40, Sq), torch.randint(0, Sq, (72,), generator=g)])
+    for h in (0, 23):
+        kf = torch.cat([t[:, h : h + 1] for t in kb_cpu], 2)
+        vf = torch.cat([t[:, h : h + 1] for t in vb_cpu], 2)
+        ro, rl = oattn.sdpa_lse_torch_cpu(q[:, h : h + 1, rows], kf, vf)
+        np.testing.assert_allclose(lse[:, h : h + 1, rows.to(cuda)].cpu().numpy(), rl.numpy(), atol=1e-3)
+        np.testing.assert_allclose(out[:, h : h + 1, rows.to(cuda)].float().cpu().numpy(), ro.float().numpy(), atol=2e-2, rtol=2e-2)

@@ -1,0 +1,115 @@
+"""Block-sparse attention: device-built runs must reproduce the mask exactly; out/LSE must match
+dense attention with -inf on the dropped tiles."""
+import numpy as np
+import pytest
+import torch
+
+import paraattention_amd
+from paraattention_amd import ops
+from oracle import attention as oattn
+from oracle import inputs
+from oracle import sparse as osparse
+
+pytestmark = pytest.mark.gpu
+
+
+def _runs_to_mask(count, ranges, nK, kv_lo, kb):
+    """Rebuild the boolean mask rows from the device's range lists (segments 1..nQ)."""
+    Hm, nseg = count.shape
+    out = np.zeros((Hm, nseg - 2, nK), dtype=bool)
+    for h in range(Hm):
+        for s in range(1, nseg - 1):
+            for r in range(count[h, s]):
+                b, e = ranges[h, s, r]
+                b, e = max(b, kv_lo), min(e, kv_lo + nK * kb)
+                if e > b:
+                    assert (b - kv_lo) % kb == 0 and (e - kv_lo) % kb == 0
+                    out[h, s - 1, (b - kv_lo) // kb : (e - kv_lo) // kb] = True
+    return out
+
+
+@pytest.mark.parametrize("Hm,nQ,nK", [(1, 1, 1), (1, 4, 7), (3, 16, 16), (24, 256, 256)])
+def test_runs_reproduce_mask_bit_exact(cuda, Hm, nQ, nK):
+    mask, _ = inputs.block_mask(Hm, nQ, nK, seed=nK)
+    kb = 128
+    count, ranges = ops.block_sparse_runs(mask.to(cuda), Skv=nK * kb)
+    count, ranges = count.cpu().numpy(), ranges.cpu().numpy()
+    assert np.array_equal(_runs_to_mask(count, ranges, nK, 0, kb), mask.numpy())
+    # and the runs are the reference's runs (sparse_attn.py:215-234)
+    for h in range(Hm):
+        for i in range(nQ):
+            want = [(s * kb, e * kb) for s, e in osparse.mask_row_runs(mask[h, i].tolist())]
+            got = [tuple(ranges[h, i + 1, r]) for r in range(count[h, i + 1])]
+            assert got == want
+    assert (count[:, 0] == 1).all() and (count[:, -1] == 1).all()
+
+
+@pytest.mark.parametrize("per_head", [False, True])
+@pytest.mark.parametrize("qb,kb", [(128, 128), (64, 32), (50, 70), (200, 24)])
+def test_small_vs_masked_dense(cuda, per_head, qb, kb):
+    B, H, nQ, nK, D = 2, 3, 5, 6, 128
+    Sq, Skv = nQ * qb, nK * kb
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=qb + kb)
+    mask, _ = inputs.block_mask(H if per_head else 1, nQ, nK, seed=1, window=0, sinks=1, density=0.5)
+    bm = mask if per_head else mask[0]
+    keep = osparse.expand_block_mask(bm.numpy(), Sq, Skv)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, keep)
+    out, lse = torch.ops.para_attn.attention_forward_block_sparse(q.to(cuda), k.to(cuda), v.to(cuda), bm.to(cuda))
+    np.testing.assert_allclose(lse.cpu().numpy(), ref_lse, atol=1e-3)
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+    if not per_head:
+        # the reference's own algorithm (runs + merges) agrees as well
+        ref2, _ = osparse.struct_sparse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), bm.numpy())
+        np.testing.assert_allclose(out.float().cpu().numpy(), ref2, atol=2e-2, rtol=2e-2)
+
+
+def test_sparse_ranges_with_dense_margins(cuda):
+    # sparse_range_query / sparse_range_key_value: dense margins on both sides (text tokens in video DiTs)
+    B, H, D = 1, 2, 128
+    Sq, Skv = 37 + 4 * 60 + 19, 20 + 5 * 48 + 33
+    q_range, kv_range = (37, 37 + 240), (20, 20 + 240)
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=77)
+    bm = torch.tensor([[1, 0, 0, 1, 1], [0, 0, 1, 0, 0], [1, 1, 1, 1, 1], [0, 1, 0, 1, 0]], dtype=torch.bool)
+    ref_out, ref_lse = osparse.struct_sparse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), bm.numpy(), None, q_range, kv_range)
+    keep = osparse.expand_block_mask(bm.numpy(), Sq, Skv, q_range, kv_range)
+    ref_out2, ref_lse2 = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, keep)
+    np.testing.assert_allclose(ref_out, ref_out2, atol=1e-9)
+    np.testing.assert_allclose(ref_lse, ref_lse2, atol=1e-9)
+    out = paraattention_amd.struct_sparse_attn_func(
+        q.to(cuda), k.to(cuda), v.to(cuda), sparse_mask=bm, sparse_range_query=q_range, sparse_range_key_value=kv_range
+    )
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+    with paraattention_amd.StructSparseAttnMode(sparse_mask=bm, sparse_range_query=q_range, sparse_range_key_value=kv_range):
+        out2 = torch.nn.functional.scaled_dot_product_attention(q.to(cuda), k.to(cuda), v.to(cuda))
+    assert torch.equal(out, out2)
+
+
+def test_row_without_kept_block(cuda):
+    # the reference asserts out on such a row (torch _SDPAMerger.results() with nothing merged);
+    # the kernel defines it: out = 0, lse = -inf
+    q, k, v = inputs.qkv(1, 1, 256, 256, 128, seed=1)
+    bm = torch.tensor([[True, False], [False, False]])
+    out, lse = torch.ops.para_attn.attention_forward_block_sparse(q.to(cuda), k.to(cuda), v.to(cuda), bm.to(cuda))
+    assert (out[:, :, 128:] == 0).all() and torch.isneginf(lse[:, :, 128:]).all()
+    assert torch.isfinite(lse[:, :, :128]).all()
+
+
+def test_config5_shape_sampled(cuda):
+    # BASELINE config 5: B1 H24 S32768 D128, 128x128 tiles, ~30% density; the oracle checks sampled
+    # query blocks of sampled heads by gathering their kept key blocks (torch CPU SDPA)
+    B, H, S, D, nb = 1, 24, 32768, 128, 256
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=0)
+    mask, density = inputs.block_mask(H, nb, nb, seed=0)
+    assert 0.28 < density < 0.32
+    out, lse = torch.ops.para_attn.attention_forward_block_sparse(q.to(cuda), k.to(cuda), v.to(cuda), mask.to(cuda))
+    g = torch.Generator().manual_seed(2)
+    for h in (0, 11, 23):
+        for i in [0, 255] + torch.randint(1, 255, (4,), generator=g).tolist():
+            rows = slice(i * 128, (i + 1) * 128)
+            idx = torch.nonzero(mask[h, i]).flatten()
+            ks = k[:, h : h + 1].reshape(1, 1, nb, 128, D)[:, :, idx].reshape(1, 1, -1, D)
+            vs = v[:, h : h + 1].reshape(1, 1, nb, 128, D)[:, :, idx].reshape(1, 1, -1, D)
+            ro, rl = oattn.sdpa_lse_torch_cpu(q[:, h : h + 1, rows], ks, vs)
+            np.testing.assert_allclose(lse[:, h : h + 1, rows].cpu().numpy(), rl.numpy(), atol=1e-3)
+            np.testing.assert_allclose(out[:, h : h + 1, rows].float().cpu().numpy(), ro.float().numpy(), atol=2e-2, rtol=2e-2)
+    assert torch.isfinite(out.float()).all()
