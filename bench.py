@@ -5,7 +5,10 @@ Prints ONE JSON line.  ``value`` is attention TFLOP/s (4*B*H*Sq*Skv*D flop per c
 resident in HBM; ``roofline`` prices the attention kernel against the bf16 dense MFMA peak;
 ``cpu_baseline`` is torch's CPU SDPA (the library routine the reference's SDPA path is checked
 against) on a bounded sample of the same workload; ``extras`` holds the bandwidth-bound kernels
-(ring merge step, FBCache reduction) against the HBM peak.
+(ring merge step, FBCache reduction) against the HBM peak and the block-sparse mode.
+
+``--only {attn,merge,fbcache,sparse}`` runs a single kernel's loop (what the rocprofv3 summaries
+under profiles/ were taken with).
 """
 import argparse
 import json
@@ -19,10 +22,12 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# measured HBM traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/), bytes
+TRAFFIC = {"attn": None, "merge": None, "fbcache": None}
 
 
 def _time_calls(fn, steps, warmup):
-    """Average milliseconds per call over ``steps`` calls, HIP events on the current stream."""
+    """(ms per call by HIP events on the launch stream, ms per call by the host clock)."""
     import torch
 
     for _ in range(warmup):
@@ -40,6 +45,109 @@ def _time_calls(fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall_ms / steps
 
 
+def _hbm(name, workload, nbytes, ms):
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {
+        "workload": workload, "bound": "hbm", "bytes_per_launch": nbytes, "ms_per_launch": round(ms, 4),
+        "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
+        "traffic": TRAFFIC.get(name),
+    }
+
+
+def bench_attn(dev, steps, warmup):
+    import torch
+
+    from oracle import inputs
+
+    B, H, S, D = 1, 3, 119056, 128
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=0, rms_norm_qk=True)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    op = torch.ops.para_attn.attention_forward_with_lse
+    ms_evt, ms_wall = _time_calls(lambda: op(qd, kd, vd), steps, warmup)
+    return (q, k, v), 4.0 * B * H * S * S * D, ms_evt, ms_wall
+
+
+def bench_merge(dev, steps=20, warmup=3):
+    import torch
+
+    # ring merge step at the ring-sweep shape: fp32 accumulator updated in place by a bf16 partial
+    B, H, S, D = 1, 24, 14882, 128
+    g = torch.Generator().manual_seed(1)
+    acc = torch.randn(B, H, S, D, generator=g).to(dev)
+    acc_l = torch.randn(B, H, S, generator=g).to(dev)
+    blk = torch.randn(B, H, S, D, generator=g).bfloat16().to(dev)
+    blk_l = torch.randn(B, H, S, generator=g).to(dev)
+    op = torch.ops.para_attn.merge_attention_lse_
+    ms, _ = _time_calls(lambda: op(acc, acc_l, blk, blk_l), steps, warmup)
+    nbytes = B * H * S * D * 10 + B * H * S * 12
+    return _hbm("merge", "ring merge step: fp32 acc [1,24,14882,128] updated in place by a bf16 partial + fp32 LSE", nbytes, ms)
+
+
+def bench_fbcache(dev, steps=20, warmup=3):
+    import torch
+
+    from oracle import inputs
+
+    prev, cur = inputs.fbcache_pair((1, 32760, 5120), seed=1234)
+    pd, cd = prev.to(dev), cur.to(dev)
+    op = torch.ops.para_attn.fbcache_residual_diff
+    ms, _ = _time_calls(lambda: op(pd, cd), steps, warmup)
+    r = _hbm("fbcache", "FBCache residual diff: bf16 [1,32760,5120] pair, threshold 0.12", 4 * prev.numel(), ms)
+    ratio = op(pd, cd).item()
+    r["ratio"] = ratio
+    r["cache_hit"] = ratio < 0.12
+    return r
+
+
+def bench_sparse(dev, steps=5, warmup=2):
+    import torch
+
+    from oracle import inputs
+
+    B, H, S, D, nb = 1, 24, 32768, 128, 256
+    q, k, v = (t.to(dev) for t in inputs.qkv(B, H, S, S, D, seed=0))
+    mask, density = inputs.block_mask(H, nb, nb, seed=0)
+    md = mask.to(dev)
+    op = torch.ops.para_attn.attention_forward_block_sparse
+    ms, _ = _time_calls(lambda: op(q, k, v, md), steps, warmup)
+    flops = 4.0 * B * H * S * S * D * density
+    tf = flops / (ms * 1e-3) / 1e12
+    return {
+        "workload": "block-sparse attention B1 H24 S32768 D128 bf16, 128x128 tiles, per-(head,q-block) mask",
+        "density": round(density, 4), "bound": "mfma", "flop_per_launch": flops, "ms_per_launch": round(ms, 4),
+        "achieved": round(tf, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4),
+    }
+
+
+def cpu_baseline(q, k, v):
+    """torch's CPU SDPA on the host cores, bounded to roughly 10-30 s of work."""
+    import torch
+
+    from oracle import attention as oattn
+
+    S, D = q.shape[2], q.shape[3]
+    cores = torch.get_num_threads()
+    ks, vs = k[:, :1].contiguous(), v[:, :1].contiguous()
+    probe = 4096
+    oattn.sdpa_lse_torch_cpu(q[:, :1, :512].contiguous(), ks, vs)  # warm the thread pool
+    t0 = time.perf_counter()
+    oattn.sdpa_lse_torch_cpu(q[:, :1, :probe].contiguous(), ks, vs)
+    per_row = (time.perf_counter() - t0) / probe
+    rows = int(min(S, max(probe, 15.0 / per_row)))  # aim at ~15 s, never more than one full head
+    qs = q[:, :1, :rows].contiguous()
+    t0 = time.perf_counter()
+    oattn.sdpa_lse_torch_cpu(qs, ks, vs)
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(4.0 * rows * S * D / dt / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"torch CPU SDPA (bf16 out + fp32 LSE): 1 of 3 heads, first {rows} of {S} query rows "
+                  f"against all {S} keys, {dt:.2f} s; rate is per unit of work, so it carries to the full call",
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -47,6 +155,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--only", choices=["attn", "merge", "fbcache", "sparse"], default=None,
+                    help="profiling aid: run just one kernel's timed loop and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (use --gpus 1)", file=sys.stderr)
@@ -56,20 +166,18 @@ def main():
 
     import paraattention_amd  # noqa: F401
     from paraattention_amd import _lib
-    from oracle import inputs
 
     _lib.load()  # no fallback: a missing library is an error
     dev = torch.device("cuda:0")
-    B, H, S, D = 1, 3, 119056, 128
-    q, k, v = inputs.qkv(B, H, S, S, D, seed=0, rms_norm_qk=True)
-    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
-    flops = 4.0 * B * H * S * S * D
 
-    op = torch.ops.para_attn.attention_forward_with_lse
-    ms_evt, ms_wall = _time_calls(lambda: op(qd, kd, vd), args.steps, args.warmup)
+    if args.only in ("merge", "fbcache", "sparse"):
+        fn = {"merge": bench_merge, "fbcache": bench_fbcache, "sparse": bench_sparse}[args.only]
+        print(json.dumps({args.only: fn(dev, args.steps, args.warmup)}))
+        return
+
+    (q, k, v), flops, ms_evt, ms_wall = bench_attn(dev, args.steps, args.warmup)
     tflops = flops / (ms_wall * 1e-3) / 1e12
     kern_tflops = flops / (ms_evt * 1e-3) / 1e12
-
     result = {
         "metric": "attn TFLOP/s & % bf16 MFMA peak at 119k-token HunyuanVideo shape; ms/call",
         "value": round(tflops, 2),
@@ -96,61 +204,20 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(kern_tflops / PEAK_BF16_TFLOPS, 4),
             "ms_per_launch": round(ms_evt, 4),
-            "traffic": None,
+            "traffic": TRAFFIC["attn"],
         },
     }
-
+    if args.only == "attn":
+        print(json.dumps(result))
+        return
     if not args.no_extras:
-        extras = {}
-        # ring merge step at the ring-sweep shape: fp32 accumulator updated in place by a bf16 partial
-        Bm, Hm, Sm = 1, 24, 14882
-        g = torch.Generator().manual_seed(1)
-        acc = torch.randn(Bm, Hm, Sm, D, generator=g).to(dev)
-        acc_l = torch.randn(Bm, Hm, Sm, generator=g).to(dev)
-        blk = torch.randn(Bm, Hm, Sm, D, generator=g).bfloat16().to(dev)
-        blk_l = torch.randn(Bm, Hm, Sm, generator=g).to(dev)
-        mop = torch.ops.para_attn.merge_attention_lse_
-        ms, _ = _time_calls(lambda: mop(acc, acc_l, blk, blk_l), 20, 3)
-        mbytes = Bm * Hm * Sm * D * 10 + Bm * Hm * Sm * 12
-        extras["merge_lse"] = {
-            "workload": "ring merge step, acc fp32 [1,24,14882,128] in place, partial bf16",
-            "bound": "hbm", "bytes_per_launch": mbytes, "ms_per_launch": round(ms, 4),
-            "achieved": round(mbytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(mbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+        result["extras"] = {
+            "merge_lse": bench_merge(dev),
+            "fbcache_residual_diff": bench_fbcache(dev),
+            "block_sparse": bench_sparse(dev),
         }
-        del acc, blk
-        # FBCache reduction at the Wan first-block residual shape
-        prev, cur = inputs.fbcache_pair((1, 32760, 5120), seed=1234)
-        pd, cd = prev.to(dev), cur.to(dev)
-        fop = torch.ops.para_attn.fbcache_residual_diff
-        ms, _ = _time_calls(lambda: fop(pd, cd), 20, 3)
-        fbytes = 4 * prev.numel()
-        extras["fbcache_residual_diff"] = {
-            "workload": "bf16 [1,32760,5120] residual pair", "ratio": fop(pd, cd).item(),
-            "bound": "hbm", "bytes_per_launch": fbytes, "ms_per_launch": round(ms, 4),
-            "achieved": round(fbytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(fbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-        }
-        del pd, cd
-        result["extras"] = extras
-
     if not args.no_cpu_baseline:
-        from oracle import attention as oattn
-
-        rows = 16384  # bounded sample: one head, the first 16384 query rows against all 119056 keys
-        cores = torch.get_num_threads()
-        qs, ks, vs = q[:, :1, :rows].contiguous(), k[:, :1].contiguous(), v[:, :1].contiguous()
-        oattn.sdpa_lse_torch_cpu(qs[:, :, :512], ks, vs)  # warm the thread pool
-        t0 = time.perf_counter()
-        oattn.sdpa_lse_torch_cpu(qs, ks, vs)
-        dt = time.perf_counter() - t0
-        result["cpu_baseline"] = {
-            "value": round(4.0 * rows * S * D / dt / 1e12, 4),
-            "unit": "TFLOP/s",
-            "cores": cores,
-            "kind": "port",
-            "sample": f"torch CPU SDPA (bf16 out + fp32 LSE), 1 head, first {rows} of {S} query rows x all {S} keys, {dt:.2f} s",
-        }
+        result["cpu_baseline"] = cpu_baseline(q, k, v)
     print(json.dumps(result))
 
 

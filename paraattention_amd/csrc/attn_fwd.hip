@@ -121,8 +121,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
   constexpr int KROWS_PER_PASS = NTHREADS / CH;
   constexpr int KPASSES = BN / KROWS_PER_PASS;
   constexpr int VGROUPS = BN / 4;  // groups of 4 key rows
-  constexpr bool V_ALL_THREADS = (NTHREADS / CH) == VGROUPS;
-  static_assert(NTHREADS / CH >= VGROUPS, "V loader mapping");
+  static_assert(64 % VGROUPS == 0 && (NTHREADS / 64) * (64 / VGROUPS) >= CH, "V loader mapping");
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t* sK = smem;                        // [2][BN][KSTRIDE]
@@ -201,9 +200,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
   u32x4 vreg[4];
   const int k_chunk = tid % CH;
   const int k_row0 = tid / CH;
-  const int v_dcol = tid % CH;
-  const int v_grp = tid / CH;  // group of 4 key rows
-  const bool v_active = V_ALL_THREADS || v_grp < VGROUPS;
+  // V loader: a wavefront covers VGROUPS(=16) row groups x 4 column chunks, so that its
+  // transposed 8-byte LDS writes (one V^T row per chunk element) spread over all banks
+  constexpr int V_CH_PER_WAVE = 64 / VGROUPS;
+  const int v_dcol = wave * V_CH_PER_WAVE + (lane % V_CH_PER_WAVE);
+  const int v_grp = lane / V_CH_PER_WAVE;  // group of 4 key rows
+  const bool v_active = v_dcol < CH;
   // position of the group inside V^T rows: swap the two low bits of the group
   const int v_grp_perm = (v_grp & ~3) | ((v_grp & 1) << 1) | ((v_grp >> 1) & 1);
 
