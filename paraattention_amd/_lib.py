@@ -9,7 +9,8 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libparaattn_hip.so")
+# PARAATTN_HIP_LIB points at another build of the same ABI (kernel experiments); default = in-tree
+LIB_PATH = os.environ.get("PARAATTN_HIP_LIB") or os.path.join(_HERE, "libparaattn_hip.so")
 
 PA_OK = 0
 PA_ERR_INVALID = -1

@@ -22,6 +22,8 @@
 // ranges per query segment, for the run loop of the reference's block-sparse
 // mode (src/para_attn/sparse_attn.py:209-240).
 
+#include <type_traits>
+
 #include "pa_common.h"
 
 namespace pa {
@@ -111,36 +113,10 @@ struct TileIter {
   }
 };
 
-template <typename T, int D, bool SPARSE>
-__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
-  typedef typename T::vec8 vec8;
-  typedef Smem<D> SM;
-  constexpr int DC = D / 16;   // contraction chunks of the first GEMM
-  constexpr int DB = D / 32;   // 32-row blocks of O^T
-  constexpr int CH = D / 8;    // 16-byte chunks per K/V row
-  constexpr int KROWS_PER_PASS = NTHREADS / CH;
-  constexpr int KPASSES = BN / KROWS_PER_PASS;
-  constexpr int VGROUPS = BN / 4;  // groups of 4 key rows
-  static_assert(64 % VGROUPS == 0 && (NTHREADS / 64) * (64 / VGROUPS) >= CH, "V loader mapping");
-
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  uint16_t* sK = smem;                        // [2][BN][KSTRIDE]
-  uint16_t* sV = smem + 2 * SM::K_ELEMS;      // [2][D][VSTRIDE]  (V^T, keys permuted)
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int l32 = lane & 31;
-  const int hh = lane >> 5;
-
-  // ---- which query rows ------------------------------------------------------
-  const int qt = blockIdx.x % p.n_qtiles;
-  const int bh = blockIdx.x / p.n_qtiles;
-  const int head = bh % p.H;
-  const int batch = bh / p.H;
-
-  int row_begin, row_end;  // query rows [row_begin, row_end) of this workgroup
-  TileIter it;
+// Which query rows a workgroup owns and which key ranges it walks.
+template <bool SPARSE>
+__device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int head, int batch,
+                                             int& row_begin, int& row_end, TileIter& it) {
   if constexpr (SPARSE) {
     int seg, tin;
     if (qt < p.tiles_left) {
@@ -180,6 +156,40 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     it.init_dense(len);
   }
 
+}
+
+template <typename T, int D, bool SPARSE>
+__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+  typedef typename T::vec8 vec8;
+  typedef Smem<D> SM;
+  constexpr int DC = D / 16;   // contraction chunks of the first GEMM
+  constexpr int DB = D / 32;   // 32-row blocks of O^T
+  constexpr int CH = D / 8;    // 16-byte chunks per K/V row
+  constexpr int KROWS_PER_PASS = NTHREADS / CH;
+  constexpr int KPASSES = BN / KROWS_PER_PASS;
+  constexpr int VGROUPS = BN / 4;  // groups of 4 key rows
+  static_assert(64 % VGROUPS == 0 && (NTHREADS / 64) * (64 / VGROUPS) >= CH, "V loader mapping");
+
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* sK = smem;                        // [2][BN][KSTRIDE]
+  uint16_t* sV = smem + 2 * SM::K_ELEMS;      // [2][D][VSTRIDE]  (V^T, keys permuted)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  // ---- which query rows ------------------------------------------------------
+  const int qt = blockIdx.x % p.n_qtiles;
+  const int bh = blockIdx.x / p.n_qtiles;
+  const int head = bh % p.H;
+  const int batch = bh / p.H;
+
+  int row_begin, row_end;  // query rows [row_begin, row_end) of this workgroup
+  TileIter it;
+  decode_block<SPARSE>(p, qt, head, batch, row_begin, row_end, it);
+
   const uint16_t* qbase = (const uint16_t*)p.q + batch * p.qs_b + head * p.qs_h;
   const uint16_t* kbase = (const uint16_t*)p.k + batch * p.ks_b + head * p.ks_h;
   const uint16_t* vbase = (const uint16_t*)p.v + batch * p.vs_b + head * p.vs_h;
@@ -193,6 +203,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const uint16_t* qp = qbase + (int64_t)r * p.qs_s + 8 * hh;
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
+    // Wait for Q here (vmcnt(0)).  Left pending, the compiler guards every first-GEMM MFMA
+    // in the loop with a vmcnt wait that, in steady state, drains the K/V prefetch instead.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
   }
 
   // ---- global -> register staging of one K/V tile ----------------------------
@@ -209,20 +222,41 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
   // position of the group inside V^T rows: swap the two low bits of the group
   const int v_grp_perm = (v_grp & ~3) | ((v_grp & 1) << 1) | ((v_grp >> 1) & 1);
 
+  // Per-thread byte offsets inside a tile (32 bit); the tile's base address is wave-uniform,
+  // so a full tile is fetched with scalar-base + vector-offset loads and no address math.
+  const int64_t ks_bytes = p.ks_s * 2, vs_bytes = p.vs_s * 2;
+  const uint32_t k_off0 = (uint32_t)(k_row0 * ks_bytes + 16 * k_chunk);
+  const uint32_t v_off0 = (uint32_t)(4 * v_grp * vs_bytes + 16 * v_dcol);
+  const char* kbytes = (const char*)kbase;
+  const char* vbytes = (const char*)vbase;
+
   auto load_tile = [&](int n0, int nvalid) {
-    const int last = n0 + nvalid - 1;
+    if (nvalid == BN) {
+      const char* kt = kbytes + (int64_t)n0 * ks_bytes;
+      const char* vt = vbytes + (int64_t)n0 * vs_bytes;
 #pragma unroll
-    for (int i = 0; i < KPASSES; ++i) {
-      int r = n0 + k_row0 + i * KROWS_PER_PASS;
-      r = r < last ? r : last;
-      kreg[i] = *(const u32x4*)(kbase + (int64_t)r * p.ks_s + 8 * k_chunk);
-    }
-    if (v_active) {
+      for (int i = 0; i < KPASSES; ++i)
+        kreg[i] = *(const u32x4*)(kt + (int64_t)i * KROWS_PER_PASS * ks_bytes + k_off0);
+      if (v_active) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int r = n0 + 4 * v_grp + i;
+        for (int i = 0; i < 4; ++i) vreg[i] = *(const u32x4*)(vt + (int64_t)i * vs_bytes + v_off0);
+      }
+    } else {
+      // ragged end of a range: rows past the end repeat the last valid row (masked later)
+      const int last = n0 + nvalid - 1;
+#pragma unroll
+      for (int i = 0; i < KPASSES; ++i) {
+        int r = n0 + k_row0 + i * KROWS_PER_PASS;
         r = r < last ? r : last;
-        vreg[i] = *(const u32x4*)(vbase + (int64_t)r * p.vs_s + 8 * v_dcol);
+        kreg[i] = *(const u32x4*)(kbytes + (int64_t)r * ks_bytes + 16 * k_chunk);
+      }
+      if (v_active) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int r = n0 + 4 * v_grp + i;
+          r = r < last ? r : last;
+          vreg[i] = *(const u32x4*)(vbytes + (int64_t)r * vs_bytes + 16 * v_dcol);
+        }
       }
     }
   };
@@ -395,6 +429,316 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// head_dim 128: the tuned kernel.
+//
+// K and V tiles (64 keys x 256 B) go from global memory straight into LDS
+// (global_load_lds_dwordx4, no register staging), row-major and unpadded, with the 16-byte
+// chunks of every row XOR-swizzled so that both the DMA writes and the fragment reads are free
+// of bank conflicts:
+//   K row r: logical chunk c is stored at chunk c ^ (r & 15)      (b128 reads down 16 rows)
+//   V row r: logical chunk c is stored at chunk c ^ (4 * (r & 3)) (transpose reads of 8x64 B)
+// The V^T operand of the second GEMM is read with ds_read_b64_tr_b16, which hands lane j of a
+// 16-lane group column j of a 4x16 block: 4 consecutive keys for one head_dim index.
+// K is fetched two tiles ahead and V one tile ahead; one workgroup barrier per tile sits between
+// the two GEMMs.  Fragment reads run one phase ahead of the MFMAs that use them, in two
+// alternating sets of 32 registers (fa / fb).
+// ---------------------------------------------------------------------------------------------
+constexpr int TILE_BYTES = BN * 256;  // one K or V tile at head_dim 128
+
+typedef __attribute__((address_space(3))) char lds_char;
+typedef const __attribute__((address_space(1))) char glb_char;
+
+template <typename T, bool SPARSE>
+__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnParams p) {
+  typedef typename T::vec8 vec8;
+  constexpr int D = 128, DC = 8, DB = 4;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  char* const sK = (char*)smem;                    // [2][64][256 B]
+  char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  const int qt = blockIdx.x % p.n_qtiles;
+  const int bh = blockIdx.x / p.n_qtiles;
+  const int head = bh % p.H;
+  const int batch = bh / p.H;
+  int row_begin, row_end;
+  TileIter itK;  // next tile whose K has to be fetched
+  decode_block<SPARSE>(p, qt, head, batch, row_begin, row_end, itK);
+  TileIter itV = itK;  // next tile whose V has to be fetched
+
+  const uint16_t* qbase = (const uint16_t*)p.q + batch * p.qs_b + head * p.qs_h;
+  const char* kbytes = (const char*)((const uint16_t*)p.k + batch * p.ks_b + head * p.ks_h);
+  const char* vbytes = (const char*)((const uint16_t*)p.v + batch * p.vs_b + head * p.vs_h);
+  const int64_t ks_bytes = p.ks_s * 2, vs_bytes = p.vs_s * 2;
+
+  // ---- Q fragment (B operand of the first GEMM) --------------------------------------------
+  const int my_row = row_begin + wave * 32 + l32;
+  const bool row_ok = my_row < row_end;
+  vec8 qf[DC];
+  {
+    int r = row_ok ? my_row : (row_end - 1);
+    const uint16_t* qp = qbase + (int64_t)r * p.qs_s + 8 * hh;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): keep Q out of the loop's wait accounting
+  }
+
+  // ---- global -> LDS copies -----------------------------------------------------------------
+  // One wave instruction moves 64 x 16 B = 4 tile rows; wave w, step i covers rows 16i+4w..+3.
+  const int dma_row = 4 * wave + (lane >> 4);  // row inside a 16-row group
+  const int dma_pc = lane & 15;                // chunk position the lane's 16 B land on
+  const uint32_t k_off0 = (uint32_t)(dma_row * ks_bytes + 16 * (dma_pc ^ (dma_row & 15)));
+  const uint32_t v_off0 = (uint32_t)(dma_row * vs_bytes + 16 * (dma_pc ^ (4 * (dma_row & 3))));
+
+  auto dma_tile = [&](const char* gbase, int64_t row_bytes, uint32_t off0, int swz_is_k, char* dst,
+                      int n0, int nvalid) {
+    lds_char* l0 = (lds_char*)dst + wave * 1024;
+    if (nvalid == BN) {
+      const char* g = gbase + (int64_t)n0 * row_bytes;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        __builtin_amdgcn_global_load_lds((glb_char*)(g + (int64_t)i * 16 * row_bytes + off0),
+                                         l0 + i * 4096, 16, 0, 0);
+    } else {
+      // ragged end of a range: rows past the end repeat the last valid row (masked later)
+      const int last = n0 + nvalid - 1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int r = n0 + 16 * i + dma_row;
+        r = r < last ? r : last;
+        const int swz = swz_is_k ? (dma_row & 15) : 4 * (dma_row & 3);
+        __builtin_amdgcn_global_load_lds((glb_char*)(gbase + (int64_t)r * row_bytes + 16 * (dma_pc ^ swz)),
+                                         l0 + i * 4096, 16, 0, 0);
+      }
+    }
+  };
+  auto dma_k = [&](int buf) {
+    int n0, nv;
+    itK.get(n0, nv);
+    dma_tile(kbytes, ks_bytes, k_off0, 1, sK + buf * TILE_BYTES, n0, nv);
+    itK.next();
+  };
+  auto dma_v = [&](int buf) {
+    int n0, nv;
+    itV.get(n0, nv);
+    dma_tile(vbytes, vs_bytes, v_off0, 0, sV + buf * TILE_BYTES, n0, nv);
+    itV.next();
+  };
+
+  // ---- fragment read addresses ---------------------------------------------------------------
+  // K (A operand of S^T = K Q^T): lane (l32, hh) reads row 32t + l32, logical chunk 2dc + hh.
+  uint32_t ka[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) ka[dc] = l32 * 256 + 16 * ((2 * dc + hh) ^ (l32 & 15));
+  // V (A operand of O^T = V^T P^T) through the transpose read: lane = (group g16, r, cq)
+  // supplies the 8 bytes at key row 4*hh + r (+ 32t + 16c + 8a), head_dim 32db + 16*dhalf + 4cq.
+  uint32_t va[DB];
+  {
+    const int g16 = lane >> 4, lg = lane & 15, r = lg >> 2, cq = lg & 3, dhalf = g16 & 1;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      va[db] = (4 * hh + r) * 256 + 16 * ((4 * db + 2 * dhalf + (cq >> 1)) ^ (4 * r)) + 8 * (cq & 1);
+  }
+  auto read_k = [&](const char* tile, int t, int dc) -> vec8 {
+    return *(const vec8*)(tile + t * 32 * 256 + ka[dc]);
+  };
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  auto read_vt = [&](const char* tile, int t, int c, int db) -> vec8 {
+    const char* a = tile + (32 * t + 16 * c) * 256 + va[db];
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + 8 * 256));
+    typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
+    s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(vec8, v);
+  };
+
+  // ---- accumulators ---------------------------------------------------------------------------
+  floatx16 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale_log2;
+
+  // ---- prologue: K0, V0, K1 in flight; first K fragments in registers --------------------------
+  int n0 = 0, cur_valid = 0, next_valid = 0;
+  bool have = itK.valid();
+  bool have_next = false;
+  vec8 fa[8], fb[8];
+  if (have) {
+    itK.get(n0, cur_valid);
+    dma_k(0);
+    dma_v(0);
+    have_next = itK.valid();
+    if (have_next) {
+      itK.get(n0, next_valid);
+      dma_k(1);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) fa[dc] = read_k(sK, 0, dc);
+  }
+
+  // One tile; PAR = which K/V buffer it lives in.
+  auto tile_step = [&](auto PAR) {
+    constexpr int par = decltype(PAR)::value;
+    const char* tK = sK + par * TILE_BYTES;
+    const char* tV = sV + par * TILE_BYTES;
+    const char* tKn = sK + (par ^ 1) * TILE_BYTES;
+
+    // ---- phase 1: S0 = K[0:32] Q^T, while the fragments of K[32:64] arrive -----------------------
+    floatx16 s0, s1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s0[r] = s1[r] = 0.f;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) fb[dc] = read_k(tK, 1, dc);
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) s0 = T::mfma32(fa[dc], qf[dc], s0);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase 2: S1 = K[32:64] Q^T ------------------------------------------------------------
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) s1 = T::mfma32(fb[dc], qf[dc], s1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // everything fetched so far has landed; after the barrier nobody still reads what comes next
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    const bool more_k = itK.valid();  // tile j+2
+    int k2_valid = 0;
+    if (more_k) {
+      itK.get(n0, k2_valid);
+      dma_k(par);
+    }
+    if (have_next) dma_v(par ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase 3: V fragments of keys 0..31 on their way, softmax meanwhile ----------------------
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) fa[cc * 4 + db] = read_vt(tV, 0, cc, db);
+
+    if (cur_valid < BN) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int n = 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (n >= cur_valid) s0[r] = -INFINITY;
+        if (n + 32 >= cur_valid) s1[r] = -INFINITY;
+      }
+    }
+    float mx = fmaxf(s0[0], s1[0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s0[r], s1[r]));
+    {
+      // other half of the row lives in lane ^ 32
+      auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+      mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    }
+    const float mx_s = mx * c;
+    if (__any(mx_s > m_run + RESCALE_SLACK)) {
+      const float m_new = fmaxf(m_run, mx_s);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+      m_run = m_new;
+    }
+    uint32_t pk0[8], pk1[8];
+    float lsum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[r], c, -m_run));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[r + 1], c, -m_run));
+      lsum += p0 + p1;
+      pk0[r >> 1] = T::pack2(p0, p1);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[r], c, -m_run));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[r + 1], c, -m_run));
+      lsum += p0 + p1;
+      pk1[r >> 1] = T::pack2(p0, p1);
+    }
+    l_run += lsum;
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase 4: O^T += V^T[:, 0:32] P^T, while the V fragments of keys 32..63 arrive -----------
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) fb[cc * 4 + db] = read_vt(tV, 1, cc, db);
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[db] = T::mfma32(fa[cc * 4 + db], bfrag, o[db]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase 5: O^T += V^T[:, 32:64] P^T, while the next tile's first K fragments arrive --------
+    if (have_next) {
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) fa[dc] = read_k(tKn, 0, dc);
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[db] = T::mfma32(fb[cc * 4 + db], bfrag, o[db]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    have = have_next;
+    cur_valid = next_valid;
+    have_next = more_k;
+    next_valid = k2_valid;
+  };
+
+  while (have) {
+    tile_step(std::integral_constant<int, 0>{});
+    if (!have) break;
+    tile_step(std::integral_constant<int, 1>{});
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------------
+  float l_tot;
+  {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+    l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  }
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  if (row_ok) {
+    uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)my_row * p.os_s;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        u32x2 w;
+        w[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
+        w[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
+        *(u32x2*)(op + 32 * db + 8 * a + 4 * hh) = w;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      p.lse[((int64_t)batch * p.H + head) * p.Sq + my_row] = lse;
+    }
+  }
+}
+
 // Turns a [Hm,nQ,nK] block mask into per-segment lists of key ranges.
 // One thread per (hm, segment); segments 0 and nQ+1 are the dense margins.
 __global__ void build_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK, int Skv,
@@ -498,19 +842,28 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
 
 template <typename T, int D, bool SPARSE>
 static int launch_attn(const AttnParams& p, hipStream_t stream) {
-  const size_t smem = Smem<D>::BYTES;
+  const void* fn;
+  size_t smem;
+  if constexpr (D == 128) {
+    fn = (const void*)attn_fwd_d128_kernel<T, SPARSE>;
+    smem = 4 * TILE_BYTES;
+  } else {
+    fn = (const void*)attn_fwd_kernel<T, D, SPARSE>;
+    smem = Smem<D>::BYTES;
+  }
   static bool attr_done = false;  // benign race: the call is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, SPARSE>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     attr_done = true;
   }
   const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
   if (nblocks == 0) return PA_OK;
-  hipLaunchKernelGGL((attn_fwd_kernel<T, D, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem,
-                     stream, p);
-  PA_CHECK_LAUNCH("attn_fwd_kernel");
+  if constexpr (D == 128)
+    hipLaunchKernelGGL((attn_fwd_d128_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+  else
+    hipLaunchKernelGGL((attn_fwd_kernel<T, D, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+  PA_CHECK_LAUNCH("attention kernel");
   return PA_OK;
 }
 
