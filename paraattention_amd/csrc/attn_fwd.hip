@@ -497,15 +497,21 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
   const uint32_t k_off0 = (uint32_t)(dma_row * ks_bytes + 16 * (dma_pc ^ (dma_row & 15)));
   const uint32_t v_off0 = (uint32_t)(dma_row * vs_bytes + 16 * (dma_pc ^ (4 * (dma_row & 3))));
 
+  // Issued as inline assembly on purpose: the compiler then keeps no account of these copies
+  // and does not make the LDS reads that follow wait for them; completion is awaited by hand
+  // (s_waitcnt vmcnt(0)) in front of the one barrier per tile.  M0 carries the LDS address of
+  // the wave's 1 KB destination; lane i's 16 bytes land at M0 + 16 i.
   auto dma_tile = [&](const char* gbase, int64_t row_bytes, uint32_t off0, int swz_is_k, char* dst,
                       int n0, int nvalid) {
-    lds_char* l0 = (lds_char*)dst + wave * 1024;
+    const uint32_t l0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)dst + wave * 1024);
     if (nvalid == BN) {
       const char* g = gbase + (int64_t)n0 * row_bytes;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        __builtin_amdgcn_global_load_lds((glb_char*)(g + (int64_t)i * 16 * row_bytes + off0),
-                                         l0 + i * 4096, 16, 0, 0);
+      for (int i = 0; i < 4; ++i) {
+        const char* gi = g + (int64_t)i * 16 * row_bytes;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(l0 + i * 4096), "v"(off0), "s"(gi) : "memory");
+      }
     } else {
       // ragged end of a range: rows past the end repeat the last valid row (masked later)
       const int last = n0 + nvalid - 1;
@@ -514,8 +520,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
         int r = n0 + 16 * i + dma_row;
         r = r < last ? r : last;
         const int swz = swz_is_k ? (dma_row & 15) : 4 * (dma_row & 3);
-        __builtin_amdgcn_global_load_lds((glb_char*)(gbase + (int64_t)r * row_bytes + 16 * (dma_pc ^ swz)),
-                                         l0 + i * 4096, 16, 0, 0);
+        const char* ga = gbase + (int64_t)r * row_bytes + 16 * (dma_pc ^ swz);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :: "s"(l0 + i * 4096), "v"(ga) : "memory");
       }
     }
   };
@@ -636,9 +643,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
         if (n + 32 >= cur_valid) s1[r] = -INFINITY;
       }
     }
-    float mx = fmaxf(s0[0], s1[0]);
+    float mx = fmaxf(s0[0], s0[1]);
 #pragma unroll
-    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s0[r], s1[r]));
+    for (int r = 2; r < 16; r += 2) mx = fmaxf(fmaxf(mx, s0[r]), s0[r + 1]);
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) mx = fmaxf(fmaxf(mx, s1[r]), s1[r + 1]);
     {
       // other half of the row lives in lane ^ 32
       auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
