@@ -664,24 +664,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
         for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
       m_run = m_new;
     }
+    // exp of keys 0..31 now; keys 32..63 are exponentiated in the shadow of the first PV MFMAs.
+    // The row sum adds the fp32 values before rounding (summing the rounded ones costs up to
+    // 3e-3 of LSE on peaked rows).
     uint32_t pk0[8], pk1[8];
     float lsum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
       float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[r], c, -m_run));
       float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[r + 1], c, -m_run));
-      lsum += p0 + p1;
       pk0[r >> 1] = T::pack2(p0, p1);
-    }
-#pragma unroll
-    for (int r = 0; r < 16; r += 2) {
-      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[r], c, -m_run));
-      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[r + 1], c, -m_run));
       lsum += p0 + p1;
-      pk1[r >> 1] = T::pack2(p0, p1);
     }
-    l_run += lsum;
-    __builtin_amdgcn_sched_barrier(0);
 
     // ---- phase 4: O^T += V^T[:, 0:32] P^T, while the V fragments of keys 32..63 arrive -----------
 #pragma unroll
@@ -695,6 +689,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 #pragma unroll
       for (int db = 0; db < DB; ++db) o[db] = T::mfma32(fa[cc * 4 + db], bfrag, o[db]);
     }
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[r], c, -m_run));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[r + 1], c, -m_run));
+      pk1[r >> 1] = T::pack2(p0, p1);
+      lsum += p0 + p1;
+    }
+    l_run += lsum;
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- phase 5: O^T += V^T[:, 32:64] P^T, while the next tile's first K fragments arrive --------

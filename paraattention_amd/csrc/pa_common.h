@@ -46,6 +46,11 @@ struct BF16 {
   }
   static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
   static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+  // acc + lo(w) + hi(w) in one instruction (v_dot2c_f32_bf16 with a vector of ones)
+  static __device__ __forceinline__ float sum2(uint32_t w, float acc) {
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, acc, false);
+  }
   static __device__ __forceinline__ floatx16 mfma32(vec8 a, vec8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -65,6 +70,10 @@ struct F16 {
   static __device__ __forceinline__ float hi(uint32_t w) {
     f16x2 r = __builtin_bit_cast(f16x2, w);
     return (float)r[1];
+  }
+  static __device__ __forceinline__ float sum2(uint32_t w, float acc) {
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, acc, false);
   }
   static __device__ __forceinline__ floatx16 mfma32(vec8 a, vec8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
