@@ -300,10 +300,22 @@ __global__ __launch_bounds__(FB_THREADS) void fbcache_apply_kernel(const void* r
   }
 }
 
-static inline int fb_grid(int64_t work_items) {
+// Grid-stride kernels here run fastest with ONE workgroup per CU (measured: 256 workgroups
+// 6.2 TB/s, 2048 workgroups 3.3 TB/s on the 671 MB reduction), each thread keeping
+// 2 x 4 16-byte loads in flight.
+static inline int fb_grid(int64_t work_items, int per_cu = 1) {
   int64_t blocks = (work_items + FB_THREADS - 1) / FB_THREADS;
   if (blocks < 1) blocks = 1;
-  const int64_t cap = 2048;  // 8 workgroups per CU
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n_cu = v;
+    else
+      n_cu = 256;
+  }
+  const int64_t cap = (int64_t)n_cu * per_cu;
   return (int)(blocks < cap ? blocks : cap);
 }
 

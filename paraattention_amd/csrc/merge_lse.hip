@@ -11,6 +11,8 @@
 
 namespace pa {
 
+constexpr int MERGE_THREADS = 512;
+
 template <int DT>
 struct Elem8;  // 8 consecutive elements of a row
 
@@ -18,8 +20,8 @@ template <>
 struct Elem8<PA_DTYPE_F32> {
   static __device__ __forceinline__ void load(const void* base, int64_t idx8, float (&x)[8]) {
     const floatx4* p = (const floatx4*)base + idx8 * 2;
-    floatx4 a = __builtin_nontemporal_load(p);
-    floatx4 b = __builtin_nontemporal_load(p + 1);
+    floatx4 a = p[0];
+    floatx4 b = p[1];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       x[i] = a[i];
@@ -38,7 +40,7 @@ struct Elem8<PA_DTYPE_F32> {
 template <>
 struct Elem8<PA_DTYPE_BF16> {
   static __device__ __forceinline__ void load(const void* base, int64_t idx8, float (&x)[8]) {
-    u32x4 w = __builtin_nontemporal_load((const u32x4*)base + idx8);
+    u32x4 w = ((const u32x4*)base)[idx8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       x[2 * i] = BF16::lo(w[i]);
@@ -56,7 +58,7 @@ struct Elem8<PA_DTYPE_BF16> {
 template <>
 struct Elem8<PA_DTYPE_F16> {
   static __device__ __forceinline__ void load(const void* base, int64_t idx8, float (&x)[8]) {
-    u32x4 w = __builtin_nontemporal_load((const u32x4*)base + idx8);
+    u32x4 w = ((const u32x4*)base)[idx8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       x[2 * i] = F16::lo(w[i]);
@@ -73,7 +75,7 @@ struct Elem8<PA_DTYPE_F16> {
 
 // One thread = 8 consecutive elements of one row.  chunks = D / 8 per row.
 template <int ACC_DT, int BLK_DT, int OUT_DT>
-__global__ __launch_bounds__(256) void merge_lse_kernel(const void* acc_out,
+__global__ __launch_bounds__(MERGE_THREADS) void merge_lse_kernel(const void* acc_out,
                                                         const float* acc_lse,
                                                         const void* __restrict__ blk_out,
                                                         const float* __restrict__ blk_lse,
@@ -116,10 +118,11 @@ template <int A, int B_, int O>
 static void launch_merge(const void* acc_out, const float* acc_lse, const void* blk_out,
                          const float* blk_lse, void* out, float* lse_out, int64_t total8, int chunks,
                          hipStream_t stream) {
-  int64_t blocks = (total8 + 255) / 256;
-  const int64_t max_blocks = 256 * 16;  // 16 resident workgroups' worth per CU, grid-stride beyond
-  if (blocks > max_blocks) blocks = max_blocks;
-  hipLaunchKernelGGL((merge_lse_kernel<A, B_, O>), dim3((unsigned)blocks), dim3(256), 0, stream,
+  // one 8-element chunk per thread, no grid cap: measured fastest (more workgroups in flight
+  // beat a capped grid-stride loop for this read+write stream)
+  int64_t blocks = (total8 + MERGE_THREADS - 1) / MERGE_THREADS;
+  if (blocks > 0x7fffffffLL) blocks = 0x7fffffffLL;
+  hipLaunchKernelGGL((merge_lse_kernel<A, B_, O>), dim3((unsigned)blocks), dim3(MERGE_THREADS), 0, stream,
                      acc_out, acc_lse, blk_out, blk_lse, out, lse_out, total8, chunks);
 }
 
