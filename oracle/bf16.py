@@ -6,9 +6,15 @@ def round_bf16(x):
     """fp32 array -> nearest bf16 value, returned as fp32 (ties to even, NaN kept)."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     u = x.view(np.uint32)
-    bias = ((u >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF)
-    r = ((u + bias) & np.uint32(0xFFFF0000)).view(np.float32)
-    return np.where(np.isnan(x), x, r).astype(np.float32)
+    r = (u >> np.uint32(16)) & np.uint32(1)
+    r += np.uint32(0x7FFF)
+    r += u
+    r &= np.uint32(0xFFFF0000)
+    r = r.view(np.float32)
+    nan = np.isnan(x)
+    if nan.any():
+        r[nan] = x[nan]
+    return r
 
 
 def round_f16(x):

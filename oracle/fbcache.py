@@ -25,7 +25,7 @@ def residual_diff_ratio(t1, t2, dtype_name="bf16"):
     mean_a = round_to(np.float32(np.sum(np.abs(a), dtype=np.float64) / n), dtype_name)
     with np.errstate(divide="ignore", invalid="ignore"):
         ratio = round_to(np.float32(mean_d) / np.float32(mean_a), dtype_name)
-    return float(ratio), float(mean_d), float(mean_a)
+    return float(np.asarray(ratio).reshape(())), float(np.asarray(mean_d).reshape(())), float(np.asarray(mean_a).reshape(()))
 
 
 def are_two_tensors_similar(t1, t2, threshold, dtype_name="bf16"):

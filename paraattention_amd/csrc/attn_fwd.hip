@@ -862,14 +862,14 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     fn = (const void*)attn_fwd_kernel<T, D, SPARSE>;
     smem = Smem<D>::BYTES;
   }
+  const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
+  if (nblocks == 0) return PA_OK;
   static bool attr_done = false;  // benign race: the call is idempotent
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     attr_done = true;
   }
-  const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
-  if (nblocks == 0) return PA_OK;
   if constexpr (D == 128)
     hipLaunchKernelGGL((attn_fwd_d128_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
   else

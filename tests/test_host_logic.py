@@ -1,0 +1,138 @@
+"""Host layer without a GPU: op names and schemas equal the reference's, fake (meta) implementations give
+the reference's output contract, config flags, cache-context gates and the no-fallback rule."""
+import os
+
+import pytest
+import torch
+
+import paraattention_amd
+from paraattention_amd import config, fbcache, ops
+
+SDPA_SCHEMA = (
+    "(Tensor query, Tensor key, Tensor value, Tensor? attn_mask=None, float dropout_p=0., "
+    "bool is_causal=False, *, float? scale=None)"
+)
+
+
+def test_op_schemas_match_reference():
+    # src/para_attn/ops/__init__.py:160-179, 204-223, 302-321: names, argument order, defaults, keyword-only scale
+    assert str(torch.ops.para_attn.attention_forward_with_lse.default._schema) == (
+        "para_attn::attention_forward_with_lse" + SDPA_SCHEMA + " -> (Tensor, Tensor)"
+    )
+    assert str(torch.ops.para_attn.attention_forward.default._schema) == "para_attn::attention_forward" + SDPA_SCHEMA + " -> Tensor"
+    assert str(torch.ops.para_attn.attention_forward_sparse_kv.default._schema) == (
+        "para_attn::attention_forward_sparse_kv" + SDPA_SCHEMA + " -> Tensor"
+    )
+    for name in ("merge_attention_lse", "merge_attention_lse_", "attention_forward_block_sparse", "fbcache_residual_diff",
+                 "fbcache_first_residual_diff", "fbcache_apply_residual"):
+        assert hasattr(torch.ops.para_attn, name)
+    assert torch.ops.para_attn.merge_attention_lse_.default._schema.arguments[0].alias_info.is_write
+
+
+def test_fake_impls_give_reference_contract():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        q = torch.empty(2, 24, 4096, 128, dtype=torch.bfloat16, device="cuda")
+        k = torch.empty(2, 24, 1024, 128, dtype=torch.bfloat16, device="cuda")
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(q, k, k)
+        # the reference's own assertions (tests/ops/test_ops.py:63-64)
+        assert out.shape == (2, 24, 4096, 128) and out.dtype == torch.bfloat16
+        assert lse.shape == (2, 24, 4096) and lse.dtype == torch.float32
+        assert torch.ops.para_attn.attention_forward(q, k, k).shape == q.shape
+        assert torch.ops.para_attn.attention_forward_sparse_kv(q, k, k).shape == q.shape
+        mo, ml = torch.ops.para_attn.merge_attention_lse(out, lse, out, lse)
+        assert mo.dtype == torch.float32 and mo.shape == out.shape and ml.shape == lse.shape
+        mo, _ = torch.ops.para_attn.merge_attention_lse(out, lse, out, lse, torch.bfloat16)
+        assert mo.dtype == torch.bfloat16
+        bm = torch.empty(32, 8, dtype=torch.bool, device="cuda")
+        so, sl = torch.ops.para_attn.attention_forward_block_sparse(q, k, k, bm)
+        assert so.shape == q.shape and sl.shape == (2, 24, 4096)
+        r = torch.ops.para_attn.fbcache_residual_diff(q, q)
+        assert r.shape == () and r.dtype == torch.bfloat16
+
+
+def test_cpu_tensors_are_refused_not_emulated():
+    # the reference asserts "Must be CUDA tensors" (src/para_attn/ops/__init__.py:123); here the dispatcher refuses
+    q = torch.randn(1, 1, 16, 128).bfloat16()
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward_with_lse(q, q, q)
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.fbcache_residual_diff(q, q)
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.merge_attention_lse(q.float(), q[..., 0].float(), q, q[..., 0].float())
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.dirname(paraattention_amd.__file__)
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text, f
+
+
+def test_config_flags_and_patch():
+    assert config.attention.allow_reduced_precision_compute in (False, True)
+    before = config.attention.allow_reduced_precision_compute
+    with config.patch(**{"attention.allow_reduced_precision_compute": not before}):
+        assert config.attention.allow_reduced_precision_compute is (not before)
+    assert config.attention.allow_reduced_precision_compute is before
+    with pytest.raises(AttributeError):
+        with config.patch(**{"attention.no_such_flag": True}):
+            pass
+
+
+def test_cache_context_gates_need_no_device():
+    x = torch.zeros(1, 4, 8)
+    with pytest.raises(AssertionError):
+        fbcache.get_can_use_cache(x)  # no context set (first_block_cache/utils.py:196-201)
+    ctx = fbcache.create_cache_context(residual_diff_threshold=0.0)
+    with fbcache.cache_context(ctx):
+        ctx.mark_step_begin()
+        assert fbcache.get_can_use_cache(x) is False  # threshold gate, utils.py:273-275
+    ctx = fbcache.create_cache_context(residual_diff_threshold=0.1, warmup_steps=2)
+    with fbcache.cache_context(ctx):
+        ctx.mark_step_begin()
+        assert ctx.get_current_step() == 0 and ctx.is_in_warmup()
+        assert fbcache.get_can_use_cache(x) is False  # warm-up gate, utils.py:271
+        ctx.mark_step_begin(); ctx.mark_step_begin()
+        assert not ctx.is_in_warmup()
+        assert fbcache.get_can_use_cache(x) is False  # nothing stored yet, utils.py:280
+    assert fbcache.get_current_cache_context() is None
+    assert fbcache.are_two_tensors_similar(x, x, threshold=0.0) is False
+    assert fbcache.are_two_tensors_similar(x, x[:, :2], threshold=0.5) is False
+    # alternating (cond / uncond) cache: buffer names and thresholds switch (utils.py:54-72, 83-92)
+    ctx = fbcache.create_cache_context(residual_diff_threshold=0.1, alter_residual_diff_threshold=0.2, enable_alter_cache=True)
+    ctx.mark_step_begin()
+    assert ctx.is_alter_cache is False and ctx.executed_steps == 1 and ctx.get_residual_diff_threshold() == 0.1
+    ctx.set_buffer("first_hidden_states_residual", 1)
+    ctx.mark_step_begin()
+    assert ctx.is_alter_cache is True and ctx.executed_steps == 1 and ctx.get_residual_diff_threshold() == 0.2
+    assert ctx.get_buffer("first_hidden_states_residual") is None
+    ctx.set_buffer("first_hidden_states_residual", 2)
+    assert ctx.buffers == {"first_hidden_states_residual": 1, "first_hidden_states_residual_alter": 2}
+
+
+def test_row_view_helper():
+    t = torch.zeros(2, 300, 512)
+    assert ops._as_rows(t) == (600, 512, 512, 1)
+    assert ops._as_rows(t[..., ::4]) == (600, 128, 512, 4)
+    assert ops._as_rows(t[:, ::2]) is None or ops._as_rows(t[:, ::2])[0] == 300  # rows no longer collapse to one stride
+    assert ops._as_rows(torch.zeros(())) == (1, 1, 1, 1)
+    assert ops._as_rows(t.transpose(0, 1)) is None
+
+
+def test_key_keep_vector():
+    B, Skv = 2, 10
+    m = torch.rand(B, Skv) < 0.5
+    assert torch.equal(ops._key_keep_vector(m[:, None, None, :], B, Skv), m)
+    assert torch.equal(ops._key_keep_vector(m[:1, None, None, :], B, Skv), m[:1].expand(B, Skv))
+    assert ops._key_keep_vector(torch.zeros(B, 1, 5, Skv, dtype=torch.bool), B, Skv) is None  # per-query mask
+    assert ops._key_keep_vector(torch.zeros(B, 1, 1, Skv), B, Skv) is None  # additive mask
+
+
+def test_merger_refuses_partial_mode():
+    m = paraattention_amd.SDPAMerger(True, 2)
+    with pytest.raises(NotImplementedError):
+        m.step(torch.zeros(1, 1, 4, 8), torch.zeros(1, 1, 4), partial=True)
