@@ -22,8 +22,9 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
-# measured HBM traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/), bytes
-TRAFFIC = {"attn": None, "merge": None, "fbcache": None}
+# HBM-side traffic per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two rocprofv3 --pmc
+# runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy; profiles/kernels_bench_workloads.md)
+TRAFFIC = {"attn": 6.528e9, "merge": 4.634e8, "fbcache": 6.710e8, "sparse": 2.132e10}
 
 
 def _time_calls(fn, steps, warmup):
@@ -116,16 +117,31 @@ def bench_sparse(dev, steps=5, warmup=2):
         "workload": "block-sparse attention B1 H24 S32768 D128 bf16, 128x128 tiles, per-(head,q-block) mask",
         "density": round(density, 4), "bound": "mfma", "flop_per_launch": flops, "ms_per_launch": round(ms, 4),
         "achieved": round(tf, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4),
+        "traffic": TRAFFIC["sparse"],
     }
 
 
+def bench_copy(dev, steps=10, warmup=2):
+    """Plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+    import torch
+
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    ms, _ = _time_calls(lambda: dst.copy_(src), steps, warmup)
+    r = _hbm("copy", "torch copy_ of 1 GiB (reads 1 GiB, writes 1 GiB)", 2 * n, ms)
+    r["read_bytes"] = n
+    r["write_bytes"] = n
+    return r
+
+
 def cpu_baseline(q, k, v):
-    """torch's CPU SDPA on the host cores, bounded to roughly 10-30 s of work."""
+    """torch's CPU SDPA on the host cores over a bounded sample (about 10-30 s) of the same workload."""
     import torch
 
     from oracle import attention as oattn
 
-    S, D = q.shape[2], q.shape[3]
+    H, S, D = q.shape[1], q.shape[2], q.shape[3]
     cores = torch.get_num_threads()
     ks, vs = k[:, :1].contiguous(), v[:, :1].contiguous()
     probe = 4096
@@ -133,18 +149,25 @@ def cpu_baseline(q, k, v):
     t0 = time.perf_counter()
     oattn.sdpa_lse_torch_cpu(q[:, :1, :probe].contiguous(), ks, vs)
     per_row = (time.perf_counter() - t0) / probe
-    rows = int(min(S, max(probe, 15.0 / per_row)))  # aim at ~15 s, never more than one full head
-    qs = q[:, :1, :rows].contiguous()
+    # whole heads while they fit in ~20 s, else a leading slice of one head's query rows
+    heads = int(min(H, 20.0 / (per_row * S)))
+    if heads >= 1:
+        qs, kk, vv, rows = q[:, :heads].contiguous(), k[:, :heads].contiguous(), v[:, :heads].contiguous(), S
+        what = f"{heads} of {H} heads, all {S} query rows"
+    else:
+        rows = int(max(probe, 15.0 / per_row))
+        heads = 1
+        qs, kk, vv = q[:, :1, :rows].contiguous(), ks, vs
+        what = f"1 of {H} heads, first {rows} of {S} query rows"
     t0 = time.perf_counter()
-    oattn.sdpa_lse_torch_cpu(qs, ks, vs)
+    oattn.sdpa_lse_torch_cpu(qs, kk, vv)
     dt = time.perf_counter() - t0
     return {
-        "value": round(4.0 * rows * S * D / dt / 1e12, 4),
+        "value": round(4.0 * heads * rows * S * D / dt / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"torch CPU SDPA (bf16 out + fp32 LSE): 1 of 3 heads, first {rows} of {S} query rows "
-                  f"against all {S} keys, {dt:.2f} s; rate is per unit of work, so it carries to the full call",
+        "sample": f"torch CPU SDPA (bf16 out + fp32 LSE): {what} against all {S} keys, {dt:.2f} s",
     }
 
 
@@ -155,7 +178,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only", choices=["attn", "merge", "fbcache", "sparse"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "fbcache", "sparse", "copy"], default=None,
                     help="profiling aid: run just one kernel's timed loop and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -170,8 +193,8 @@ def main():
     _lib.load()  # no fallback: a missing library is an error
     dev = torch.device("cuda:0")
 
-    if args.only in ("merge", "fbcache", "sparse"):
-        fn = {"merge": bench_merge, "fbcache": bench_fbcache, "sparse": bench_sparse}[args.only]
+    if args.only in ("merge", "fbcache", "sparse", "copy"):
+        fn = {"merge": bench_merge, "fbcache": bench_fbcache, "sparse": bench_sparse, "copy": bench_copy}[args.only]
         print(json.dumps({args.only: fn(dev, args.steps, args.warmup)}))
         return
 
@@ -198,7 +221,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "attn_fwd_kernel<BF16,128,dense>",
+            "kernel": "pa::attn_fwd_d128_kernel<pa::BF16, false>",
             "achieved": round(kern_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",

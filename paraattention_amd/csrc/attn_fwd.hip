@@ -751,29 +751,34 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 }
 
 // Turns a [Hm,nQ,nK] block mask into per-segment lists of key ranges.
-// One thread per (hm, segment); segments 0 and nQ+1 are the dense margins.
-__global__ void build_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK, int Skv,
-                                  int kv_lo, int kv_block, int cap, int32_t* ws) {
+// One wavefront per (hm, segment): the lanes read 64 mask bytes at a time and vote them into a
+// bit word; lane 0 then walks the words and emits the runs of kept blocks (the scan of
+// src/para_attn/sparse_attn.py:215-234), merged with the dense key margins where they touch.
+// Segments 0 and nQ+1 are the dense query margins.
+__global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK,
+                                                        int Skv, int kv_lo, int kv_block, int cap,
+                                                        int32_t* ws) {
   const int nseg = nQ + 2;
-  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= Hm * nseg) return;
+  const int idx = blockIdx.x;  // grid = Hm * nseg
+  const int lane = threadIdx.x;
   const int hm = idx / nseg;
   const int seg = idx % nseg;
   int32_t* cnt = ws + idx;
   int32_t* rg = ws + (size_t)Hm * nseg + (size_t)idx * cap * 2;
-  int n = 0;
   if (seg == 0 || seg == nQ + 1) {
-    if (Skv > 0) {
-      rg[0] = 0;
-      rg[1] = Skv;
-      n = 1;
+    if (lane == 0) {
+      if (Skv > 0) {
+        rg[0] = 0;
+        rg[1] = Skv;
+      }
+      *cnt = Skv > 0 ? 1 : 0;
     }
-    *cnt = n;
     return;
   }
   const uint8_t* row = mask + ((size_t)hm * nQ + (seg - 1)) * nK;
   const int kv_hi = kv_lo + nK * kv_block;
-  int cur_b = -1, cur_e = -1;  // open range
+  int n = 0;
+  int cur_b = -1, cur_e = -1;  // open range (lane 0 only)
   auto push = [&](int b, int e) {
     if (e <= b) return;
     if (cur_e == b) {
@@ -788,25 +793,45 @@ __global__ void build_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK, i
       cur_e = e;
     }
   };
-  push(0, kv_lo);
-  int j = 0;
-  while (j < nK) {
-    if (!row[j]) {
-      ++j;
-      continue;
+  if (lane == 0) push(0, kv_lo);
+  int run_start = -1;  // block index where the current run of kept blocks began, -1 = none
+  for (int base = 0; base < nK; base += 64) {
+    const int j = base + lane;
+    const bool keep = j < nK && row[j] != 0;
+    uint64_t bits = __ballot(keep);
+    if (lane == 0) {
+      int pos = 0;  // bits below pos are consumed
+      while (pos < 64) {
+        if (run_start < 0) {
+          if (bits == 0) break;
+          const int z = __builtin_ctzll(bits);  // skip dropped blocks
+          pos += z;
+          bits >>= z;  // z <= 63 because bits != 0
+          run_start = base + pos;
+        } else {
+          const uint64_t inv = ~bits;
+          const int o = inv == 0 ? 64 : __builtin_ctzll(inv);
+          const int ones = o < 64 - pos ? o : 64 - pos;  // kept blocks in a row, within this word
+          pos += ones;
+          bits = ones < 64 ? bits >> ones : 0;
+          if (pos < 64) {  // the run ended inside this word
+            push(kv_lo + run_start * kv_block, kv_lo + (base + pos) * kv_block);
+            run_start = -1;
+          }
+        }
+      }
     }
-    int e = j + 1;
-    while (e < nK && row[e]) ++e;
-    push(kv_lo + j * kv_block, kv_lo + e * kv_block);
-    j = e;
   }
-  push(kv_hi, Skv);
-  if (cur_e > cur_b) {
-    rg[2 * n] = cur_b;
-    rg[2 * n + 1] = cur_e;
-    ++n;
+  if (lane == 0) {
+    if (run_start >= 0) push(kv_lo + run_start * kv_block, kv_hi);
+    push(kv_hi, Skv);
+    if (cur_e > cur_b) {
+      rg[2 * n] = cur_b;
+      rg[2 * n + 1] = cur_e;
+      ++n;
+    }
+    *cnt = n;
   }
-  *cnt = n;
 }
 
 }  // namespace pa
@@ -922,7 +947,7 @@ extern "C" int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int 
     PA_FAIL(PA_ERR_WORKSPACE, "runs workspace too small");
   const int total = Hm * (nQ + 2);
   const int cap = nK / 2 + 3;
-  hipLaunchKernelGGL(build_runs_kernel, dim3((total + 63) / 64), dim3(64), 0, (hipStream_t)stream,
+  hipLaunchKernelGGL(build_runs_kernel, dim3(total), dim3(64), 0, (hipStream_t)stream,
                      block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, cap, runs_ws);
   PA_CHECK_LAUNCH("build_runs_kernel");
   return PA_OK;

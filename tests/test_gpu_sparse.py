@@ -44,6 +44,25 @@ def test_runs_reproduce_mask_bit_exact(cuda, Hm, nQ, nK):
     assert (count[:, 0] == 1).all() and (count[:, -1] == 1).all()
 
 
+def test_runs_word_boundaries(cuda):
+    # rows that exercise the 64-block voting words: kept block at bit 63, runs crossing words, all kept, none kept
+    nK = 200
+    rows = torch.zeros(8, nK, dtype=torch.bool)
+    rows[0, 63] = True
+    rows[1, 60:70] = True
+    rows[2, :] = True
+    rows[4, 0] = True; rows[4, 127:129] = True; rows[4, 199] = True
+    rows[5, 64:128] = True
+    rows[6, 1::2] = True
+    rows[7, 63:65] = True; rows[7, 191:193] = True
+    count, ranges = ops.block_sparse_runs(rows[None].to(cuda), Skv=nK * 16)
+    count, ranges = count.cpu().numpy(), ranges.cpu().numpy()
+    for i in range(8):
+        want = [(s * 16, e * 16) for s, e in osparse.mask_row_runs(rows[i].tolist())]
+        got = [tuple(ranges[0, i + 1, r]) for r in range(count[0, i + 1])]
+        assert got == want, i
+
+
 @pytest.mark.parametrize("per_head", [False, True])
 @pytest.mark.parametrize("qb,kb", [(128, 128), (64, 32), (50, 70), (200, 24)])
 def test_small_vs_masked_dense(cuda, per_head, qb, kb):
