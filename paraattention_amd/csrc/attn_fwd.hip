@@ -446,6 +446,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
 // alternating sets of 32 registers (fa / fb).
 // ---------------------------------------------------------------------------------------------
 constexpr int TILE_BYTES = BN * 256;  // one K or V tile at head_dim 128
+// Buffer offset that is out of range for every tensor the pipelined kernel accepts (its host side
+// refuses K or V extents of this size or more and takes the kernel above instead).
+constexpr uint32_t PIPE_OOB = 0xfffff000u;
 
 typedef __attribute__((address_space(3))) char lds_char;
 typedef const __attribute__((address_space(1))) char glb_char;
@@ -750,6 +753,334 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// head_dim 128, two-tile software pipeline (the kernel used unless K or V spans 4 GiB or more).
+//
+// Same tile layout in LDS as the kernel above (row-major, XOR-swizzled chunks, LDS-DMA fills,
+// transpose reads for V).  What differs is the order of work inside a wavefront.  Iteration j
+// holds two score tiles, S(j) being exponentiated and S(j+1) being produced:
+//
+//   barrier            K(j+1) and V(j) have landed; everybody is done with iteration j-1
+//   rare rescale of O  from the row maximum of S(j), taken one iteration earlier
+//   stage A  16 x { MFMA of S(j+1) = K(j+1) Q^T ; one LDS-DMA issue for K(j+2) / V(j+1) (first 8) ;
+//                   refill of the consumed fragment slot ; exp2 / sum / pack of two scores of S(j) }
+//   stage B  16 x { MFMA of O^T += V(j)^T P(j)^T ; refill ; part of the row maximum of S(j+1) }
+//
+// so exponentials, the issue stalls of the tile copies and the row maximum all sit in the shadow
+// of MFMAs of the same wavefront.  Every iteration runs the same code: a tile that does not exist
+// is fetched out of bounds (the buffer descriptor returns zeros) and its scores are never used.
+// ---------------------------------------------------------------------------------------------
+template <typename T, bool SPARSE>
+__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const AttnParams p) {
+  typedef typename T::vec8 vec8;
+  constexpr int DC = 8, DB = 4;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  char* const sK = (char*)smem;                    // [2][64][256 B]
+  char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  const int qt = blockIdx.x % p.n_qtiles;
+  const int bh = blockIdx.x / p.n_qtiles;
+  const int head = bh % p.H;
+  const int batch = bh / p.H;
+  int row_begin, row_end;
+  TileIter it;
+  decode_block<SPARSE>(p, qt, head, batch, row_begin, row_end, it);
+
+  const uint16_t* qbase = (const uint16_t*)p.q + batch * p.qs_b + head * p.qs_h;
+  const char* kbytes = (const char*)((const uint16_t*)p.k + batch * p.ks_b + head * p.ks_h);
+  const char* vbytes = (const char*)((const uint16_t*)p.v + batch * p.vs_b + head * p.vs_h);
+  const uint32_t ks_bytes = (uint32_t)(p.ks_s * 2), vs_bytes = (uint32_t)(p.vs_s * 2);
+
+  // ---- Q fragment (B operand of the first GEMM) --------------------------------------------
+  const int my_row = row_begin + wave * 32 + l32;
+  const bool row_ok = my_row < row_end;
+  vec8 qf[DC];
+  {
+    int r = row_ok ? my_row : (row_end - 1);
+    const uint16_t* qp = qbase + (int64_t)r * p.qs_s + 8 * hh;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): keep Q out of the loop's wait accounting
+  }
+
+  // ---- global -> LDS copies: raw buffer loads with the LDS bit ---------------------------------
+  // The descriptor bounds the whole K (V) of this batch and head, so rows past the last key come
+  // back as zeros instead of needing an address clamp.  One wave instruction moves 4 tile rows;
+  // wave w, step i covers rows 16i+4w..+3; lane l lands on chunk l%16 of row l/16 and fetches
+  // the logical chunk that the swizzle maps there.  Inline assembly on purpose: the compiler
+  // keeps no account of these copies, so LDS reads that follow do not wait for them; completion
+  // is awaited by hand (vmcnt(0)) in front of the barrier.
+  auto make_rsrc = [&](const char* base, uint32_t row_bytes) {
+    u32x4 r;
+    const uint64_t a = (uint64_t)base;
+    const uint64_t nbytes = (uint64_t)(p.Skv - 1) * row_bytes + 256;  // start of the last row + one row
+    r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+    r[2] = __builtin_amdgcn_readfirstlane((uint32_t)nbytes);
+    r[3] = 0x00020000u;
+    return r;
+  };
+  const u32x4 krs = make_rsrc(kbytes, ks_bytes);
+  const u32x4 vrs = make_rsrc(vbytes, vs_bytes);
+  const int dma_row = 4 * wave + (lane >> 4);
+  const int dma_pc = lane & 15;
+  const uint32_t k_off0 = dma_row * ks_bytes + 16 * (dma_pc ^ (dma_row & 15));
+  const uint32_t v_off0 = dma_row * vs_bytes + 16 * (dma_pc ^ (4 * (dma_row & 3)));
+  const uint32_t lds_k = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sK + wave * 1024);
+  const uint32_t lds_v = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sV + wave * 1024);
+  constexpr uint32_t OOB = PIPE_OOB;  // first key of a tile that does not exist; also its soffset
+  // i-th of the four copy instructions of the K (V) tile starting at key n0, into buffer `buf`
+  auto dma_k1 = [&](int buf, uint32_t n0, int i) {
+    const uint32_t soff = n0 == OOB ? OOB : (n0 + 16 * i) * ks_bytes;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_k + buf * TILE_BYTES + i * 4096), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
+  };
+  auto dma_v1 = [&](int buf, uint32_t n0, int i) {
+    const uint32_t soff = n0 == OOB ? OOB : (n0 + 16 * i) * vs_bytes;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_v + buf * TILE_BYTES + i * 4096), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
+  };
+
+  // ---- fragment read addresses (as in the kernel above) -------------------------------------------
+  uint32_t ka[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) ka[dc] = l32 * 256 + 16 * ((2 * dc + hh) ^ (l32 & 15));
+  uint32_t va[DB];
+  {
+    const int g16 = lane >> 4, lg = lane & 15, r = lg >> 2, cq = lg & 3, dhalf = g16 & 1;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      va[db] = (4 * hh + r) * 256 + 16 * ((4 * db + 2 * dhalf + (cq >> 1)) ^ (4 * r)) + 8 * (cq & 1);
+  }
+  auto read_k = [&](const char* tile, int t, int dc) -> vec8 {
+    return *(const vec8*)(tile + t * 32 * 256 + ka[dc]);
+  };
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  auto read_vt = [&](const char* tile, int t, int c, int db) -> vec8 {
+    const char* a = tile + (32 * t + 16 * c) * 256 + va[db];
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + 8 * 256));
+    typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
+    s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(vec8, v);
+  };
+
+  // ---- accumulators ---------------------------------------------------------------------------
+  floatx16 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale_log2;
+
+  // window of tiles j (being consumed), j+1 and j+2: (first key or OOB, valid keys)
+  uint32_t n_cur, n_nxt, n_nx2;
+  int v_cur, v_nxt, v_nx2;
+  auto pull = [&](uint32_t& n0, int& nv) {
+    if (it.valid()) {
+      int a, b;
+      it.get(a, b);
+      it.next();
+      n0 = (uint32_t)a;
+      nv = b;
+    } else {
+      n0 = OOB;
+      nv = 0;
+    }
+  };
+  pull(n_cur, v_cur);
+  pull(n_nxt, v_nxt);
+  pull(n_nx2, v_nx2);
+  bool have = n_cur != OOB;
+
+  // -inf on the keys past the end of a ragged tile: register r of this lane is key
+  // 8*(r/4) + r%4 + 4*hh of the first half (+32 for the second); constants against one per-lane
+  // limit, so nothing per register stays live across the loop
+  auto mask_tail = [&](floatx16& a0, floatx16& a1, int nvalid) {
+    const int lim = nvalid - 4 * hh;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (8 * (r >> 2) + (r & 3) >= lim) a0[r] = -INFINITY;
+      if (8 * (r >> 2) + (r & 3) + 32 >= lim) a1[r] = -INFINITY;
+    }
+  };
+  // other half of a query row lives in lane ^ 32
+  auto across = [&](float x) {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+  };
+
+  vec8 f[8];          // ring of 8 operand fragments: a slot is refilled as soon as its MFMA has issued
+  floatx16 sn0, sn1;  // S(j+1) (keys 0..31, 32..63); it is S(j) at the top of the next iteration
+  float mx = 0.f;     // row maximum of S(j), masked, unscaled
+#pragma unroll
+  for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+
+  // ---- prologue: K0, V0, K1 copies; S(0) and its row maximum ---------------------------------
+  if (have) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_k1(0, n_cur, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_v1(0, n_cur, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_k1(1, n_nxt, i);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(sK, 0, dc);
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+      sn0 = T::mfma32(f[dc], qf[dc], sn0);
+      f[dc] = read_k(sK, 1, dc);
+    }
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
+    if (v_cur < BN) mask_tail(sn0, sn1, v_cur);
+    float m2 = fmaxf(sn0[0], sn1[0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
+    mx = across(m2);
+  }
+
+  // One iteration; PAR = buffer of tile j (K(j+1) sits in the other K buffer).
+  auto tile_step = [&](auto PAR) {
+    constexpr int par = decltype(PAR)::value;
+    const char* tV = sV + par * TILE_BYTES;
+    const char* tKn = sK + (par ^ 1) * TILE_BYTES;
+    floatx16 c0 = sn0, c1 = sn1;  // S(j)
+
+    // everything fetched so far has landed; after the barrier nobody still reads what comes next
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+
+    // first fragments of K(j+1) on their way while the maximum is settled
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, 0, dc);
+
+    const float mx_s = mx * c;
+    if (__any(mx_s > m_run + RESCALE_SLACK)) {
+      const float m_new = fmaxf(m_run, mx_s);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+      m_run = m_new;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- stage A ---------------------------------------------------------------------------------
+    // The row sum adds the fp32 values before rounding (summing the rounded ones costs up to 3e-3
+    // of LSE on peaked rows).
+    uint32_t pk0[8], pk1[8];
+    float lsum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      sn0 = T::mfma32(f[g], qf[g], sn0);
+      if (g < 4) dma_k1(par, n_nx2, g);    // K(j+2) takes the buffer K(j) has left
+      else dma_v1(par ^ 1, n_nxt, g - 4);  // V(j+1) takes the buffer V(j-1) has left
+      f[g] = read_k(tKn, 1, g);
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(c0[2 * g], c, -m_run));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(c0[2 * g + 1], c, -m_run));
+      lsum += p0 + p1;
+      pk0[g] = T::pack2(p0, p1);
+      __builtin_amdgcn_sched_barrier(0);  // keep the groups in this order
+    }
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      sn1 = T::mfma32(f[g], qf[g], sn1);
+      f[g] = read_vt(tV, 0, g >> 2, g & 3);  // V(j), keys 0..31, takes the slot over
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(c1[2 * g], c, -m_run));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(c1[2 * g + 1], c, -m_run));
+      lsum += p0 + p1;
+      pk1[g] = T::pack2(p0, p1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    l_run += lsum;
+    if (v_nxt < BN) mask_tail(sn0, sn1, v_nxt);  // ragged (or absent) tile j+1
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- stage B ---------------------------------------------------------------------------------
+    float mxa = fmaxf(sn0[0], sn0[1]), mxb = fmaxf(sn1[0], sn1[1]);
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int g = cc * 4 + db;
+        o[db] = T::mfma32(f[g], bfrag, o[db]);
+        f[g] = read_vt(tV, 1, cc, db);  // keys 32..63
+        if (g > 0) mxa = fmaxf(fmaxf(mxa, sn0[2 * g]), sn0[2 * g + 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int g = cc * 4 + db;
+        o[db] = T::mfma32(f[g], bfrag, o[db]);
+        if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    mx = across(fmaxf(mxa, mxb));
+
+    // slide the tile window
+    n_cur = n_nxt;
+    v_cur = v_nxt;
+    n_nxt = n_nx2;
+    v_nxt = v_nx2;
+    pull(n_nx2, v_nx2);
+    have = n_cur != OOB;
+  };
+
+  while (have) {
+    tile_step(std::integral_constant<int, 0>{});
+    if (!have) break;
+    tile_step(std::integral_constant<int, 1>{});
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------------
+  float l_tot;
+  {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+    l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  }
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  if (row_ok) {
+    uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)my_row * p.os_s;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        u32x2 w;
+        w[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
+        w[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
+        *(u32x2*)(op + 32 * db + 8 * a + 4 * hh) = w;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      p.lse[((int64_t)batch * p.H + head) * p.Sq + my_row] = lse;
+    }
+  }
+}
+
 // Turns a [Hm,nQ,nK] block mask into per-segment lists of key ranges.
 // One wavefront per (hm, segment): the lanes read 64 mask bytes at a time and vote them into a
 // bit word; lane 0 then walks the words and emits the runs of kept blocks (the scan of
@@ -878,27 +1209,34 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
 
 template <typename T, int D, bool SPARSE>
 static int launch_attn(const AttnParams& p, hipStream_t stream) {
+  const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
+  if (nblocks == 0) return PA_OK;
+  // the pipelined kernel addresses K and V through 32-bit buffer offsets
+  const bool pipe = D == 128 && p.Skv > 0 && (uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 < PIPE_OOB &&
+                    (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 < PIPE_OOB;
   const void* fn;
   size_t smem;
   if constexpr (D == 128) {
-    fn = (const void*)attn_fwd_d128_kernel<T, SPARSE>;
+    fn = pipe ? (const void*)attn_fwd_d128_pipe_kernel<T, SPARSE> : (const void*)attn_fwd_d128_kernel<T, SPARSE>;
     smem = 4 * TILE_BYTES;
   } else {
     fn = (const void*)attn_fwd_kernel<T, D, SPARSE>;
     smem = Smem<D>::BYTES;
   }
-  const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
-  if (nblocks == 0) return PA_OK;
-  static bool attr_done = false;  // benign race: the call is idempotent
-  if (!attr_done) {
+  static bool attr_done[2] = {false, false};  // benign race: the call is idempotent
+  if (!attr_done[pipe]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_done = true;
+    attr_done[pipe] = true;
   }
-  if constexpr (D == 128)
-    hipLaunchKernelGGL((attn_fwd_d128_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
-  else
+  if constexpr (D == 128) {
+    if (pipe)
+      hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+    else
+      hipLaunchKernelGGL((attn_fwd_d128_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+  } else {
     hipLaunchKernelGGL((attn_fwd_kernel<T, D, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+  }
   PA_CHECK_LAUNCH("attention kernel");
   return PA_OK;
 }
