@@ -980,10 +980,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const A
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage A ---------------------------------------------------------------------------------
-    // The row sum adds the fp32 values before rounding (summing the rounded ones costs up to 3e-3
-    // of LSE on peaked rows).
+    // The 32 scores of S(j) per lane are exponentiated 24 in stage A and 8 in the first half of
+    // stage B (P of keys 32..63 is only needed by the last 8 MFMAs), which keeps the VALU work
+    // per MFMA below the MFMA's own 32 cycles.  The row sum adds the fp32 values before rounding
+    // (summing the rounded ones costs up to 3e-3 of LSE on peaked rows).
     uint32_t pk0[8], pk1[8];
     float lsum = 0.f;
+    auto expo = [&](const floatx16& cs, uint32_t* pk, int i) {  // scores 2i, 2i+1 -> packed pair i
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cs[2 * i], c, -m_run));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cs[2 * i + 1], c, -m_run));
+      lsum += p0 + p1;
+      pk[i] = T::pack2(p0, p1);
+    };
 #pragma unroll
     for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
 #pragma unroll
@@ -992,23 +1000,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const A
       if (g < 4) dma_k1(par, n_nx2, g);    // K(j+2) takes the buffer K(j) has left
       else dma_v1(par ^ 1, n_nxt, g - 4);  // V(j+1) takes the buffer V(j-1) has left
       f[g] = read_k(tKn, 1, g);
-      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(c0[2 * g], c, -m_run));
-      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(c0[2 * g + 1], c, -m_run));
-      lsum += p0 + p1;
-      pk0[g] = T::pack2(p0, p1);
+      expo(c0, pk0, g);
       __builtin_amdgcn_sched_barrier(0);  // keep the groups in this order
     }
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
       sn1 = T::mfma32(f[g], qf[g], sn1);
       f[g] = read_vt(tV, 0, g >> 2, g & 3);  // V(j), keys 0..31, takes the slot over
-      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(c1[2 * g], c, -m_run));
-      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(c1[2 * g + 1], c, -m_run));
-      lsum += p0 + p1;
-      pk1[g] = T::pack2(p0, p1);
+      if (g < 4) expo(c1, pk1, g);
       __builtin_amdgcn_sched_barrier(0);
     }
-    l_run += lsum;
     if (v_nxt < BN) mask_tail(sn0, sn1, v_nxt);  // ragged (or absent) tile j+1
     __builtin_amdgcn_sched_barrier(0);
 
@@ -1023,10 +1024,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const A
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
         f[g] = read_vt(tV, 1, cc, db);  // keys 32..63
-        if (g > 0) mxa = fmaxf(fmaxf(mxa, sn0[2 * g]), sn0[2 * g + 1]);
+        if (g < 4) expo(c1, pk1, 4 + g);
+        else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
+        else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    l_run += lsum;
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
