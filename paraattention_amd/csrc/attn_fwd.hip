@@ -22,6 +22,8 @@
 // ranges per query segment, for the run loop of the reference's block-sparse
 // mode (src/para_attn/sparse_attn.py:209-240).
 
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "pa_common.h"
@@ -50,6 +52,8 @@ struct AttnParams {
   int64_t os_b, os_h, os_s;
   float scale_log2;  // scale * log2(e), > 0
   int n_qtiles;      // workgroups per (batch, head)
+  int bm;            // query rows per workgroup (32 per wavefront)
+  int pipe;          // head_dim 128: 1 = pipelined kernel, 0 = the one without 32-bit offset limits
   const int32_t* kv_len;  // dense: optional per-batch key count
   // block-sparse only
   const int32_t* runs;  // count[Hm*nSeg] then range[Hm*nSeg][cap][2]
@@ -122,7 +126,7 @@ __device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int he
     if (qt < p.tiles_left) {
       seg = 0;
       tin = qt;
-      row_begin = tin * BM;
+      row_begin = tin * p.bm;
       row_end = p.q_lo;
     } else {
       int r = qt - p.tiles_left;
@@ -130,24 +134,24 @@ __device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int he
       if (blk < p.nQ) {
         seg = 1 + blk;
         tin = r - blk * p.tiles_per_block;
-        row_begin = p.q_lo + blk * p.q_block + tin * BM;
+        row_begin = p.q_lo + blk * p.q_block + tin * p.bm;
         row_end = p.q_lo + (blk + 1) * p.q_block;
       } else {
         seg = p.nQ + 1;
         tin = r - p.nQ * p.tiles_per_block;
-        row_begin = p.q_lo + p.nQ * p.q_block + tin * BM;
+        row_begin = p.q_lo + p.nQ * p.q_block + tin * p.bm;
         row_end = p.Sq;
       }
     }
-    if (row_end > row_begin + BM) row_end = row_begin + BM;
+    if (row_end > row_begin + p.bm) row_end = row_begin + p.bm;
     const int nseg = p.nQ + 2;
     const int hm = p.Hm == 1 ? 0 : head;
     const int sidx = hm * nseg + seg;
     const int cnt = p.runs[sidx];
     it.init_list(p.runs + (size_t)p.Hm * nseg + (size_t)sidx * p.cap * 2, cnt);
   } else {
-    row_begin = qt * BM;
-    row_end = row_begin + BM < p.Sq ? row_begin + BM : p.Sq;
+    row_begin = qt * p.bm;
+    row_end = row_begin + p.bm < p.Sq ? row_begin + p.bm : p.Sq;
     int len = p.Skv;
     if (p.kv_len) {
       int kl = p.kv_len[batch];
@@ -771,10 +775,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 // of MFMAs of the same wavefront.  Every iteration runs the same code: a tile that does not exist
 // is fetched out of bounds (the buffer descriptor returns zeros) and its scores are never used.
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool SPARSE>
-__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const AttnParams p) {
+template <typename T, bool SPARSE, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
   constexpr int DC = 8, DB = 4;
+  constexpr int IPW = 16 / NW;  // copy instructions per wavefront and K (V) tile
+  constexpr int RS = 4 * NW;    // tile rows between two of them
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                    // [2][64][256 B]
   char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
@@ -813,7 +819,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const A
   // ---- global -> LDS copies: raw buffer loads with the LDS bit ---------------------------------
   // The descriptor bounds the whole K (V) of this batch and head, so rows past the last key come
   // back as zeros instead of needing an address clamp.  One wave instruction moves 4 tile rows;
-  // wave w, step i covers rows 16i+4w..+3; lane l lands on chunk l%16 of row l/16 and fetches
+  // wave w, step i covers rows RS*i+4w..+3; lane l lands on chunk l%16 of row l/16 and fetches
   // the logical chunk that the swizzle maps there.  Inline assembly on purpose: the compiler
   // keeps no account of these copies, so LDS reads that follow do not wait for them; completion
   // is awaited by hand (vmcnt(0)) in front of the barrier.
@@ -838,14 +844,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const A
   constexpr uint32_t OOB = PIPE_OOB;  // first key of a tile that does not exist; also its soffset
   // i-th of the four copy instructions of the K (V) tile starting at key n0, into buffer `buf`
   auto dma_k1 = [&](int buf, uint32_t n0, int i) {
-    const uint32_t soff = n0 == OOB ? OOB : (n0 + 16 * i) * ks_bytes;
+    const uint32_t soff = n0 == OOB ? OOB : (n0 + RS * i) * ks_bytes;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds_k + buf * TILE_BYTES + i * 4096), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
+                 :: "s"(lds_k + buf * TILE_BYTES + i * (RS * 256)), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
   };
   auto dma_v1 = [&](int buf, uint32_t n0, int i) {
-    const uint32_t soff = n0 == OOB ? OOB : (n0 + 16 * i) * vs_bytes;
+    const uint32_t soff = n0 == OOB ? OOB : (n0 + RS * i) * vs_bytes;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds_v + buf * TILE_BYTES + i * 4096), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
+                 :: "s"(lds_v + buf * TILE_BYTES + i * (RS * 256)), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
   };
 
   // ---- fragment read addresses (as in the kernel above) -------------------------------------------
@@ -928,11 +934,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const A
   // ---- prologue: K0, V0, K1 copies; S(0) and its row maximum ---------------------------------
   if (have) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma_k1(0, n_cur, i);
+    for (int i = 0; i < IPW; ++i) dma_k1(0, n_cur, i);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma_v1(0, n_cur, i);
+    for (int i = 0; i < IPW; ++i) dma_v1(0, n_cur, i);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma_k1(1, n_nxt, i);
+    for (int i = 0; i < IPW; ++i) dma_k1(1, n_nxt, i);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 #pragma unroll
@@ -997,8 +1003,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_pipe_kernel(const A
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
       sn0 = T::mfma32(f[g], qf[g], sn0);
-      if (g < 4) dma_k1(par, n_nx2, g);    // K(j+2) takes the buffer K(j) has left
-      else dma_v1(par ^ 1, n_nxt, g - 4);  // V(j+1) takes the buffer V(j-1) has left
+      if (g < IPW) dma_k1(par, n_nx2, g);                      // K(j+2) takes the buffer K(j) has left
+      else if (g < 2 * IPW) dma_v1(par ^ 1, n_nxt, g - IPW);  // V(j+1) takes the buffer V(j-1) has left
       f[g] = read_k(tKn, 1, g);
       expo(c0, pk0, g);
       __builtin_amdgcn_sched_barrier(0);  // keep the groups in this order
@@ -1209,33 +1215,37 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.kv_len = nullptr;
   p.runs = nullptr;
   p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.tiles_left = 0; p.tiles_per_block = 0;
+  p.bm = BM; p.pipe = 0;
 }
 
 template <typename T, int D, bool SPARSE>
 static int launch_attn(const AttnParams& p, hipStream_t stream) {
   const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
   if (nblocks == 0) return PA_OK;
-  // the pipelined kernel addresses K and V through 32-bit buffer offsets
-  const bool pipe = D == 128 && p.Skv > 0 && (uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 < PIPE_OOB &&
-                    (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 < PIPE_OOB;
   const void* fn;
   size_t smem;
+  int slot;
   if constexpr (D == 128) {
-    fn = pipe ? (const void*)attn_fwd_d128_pipe_kernel<T, SPARSE> : (const void*)attn_fwd_d128_kernel<T, SPARSE>;
     smem = 4 * TILE_BYTES;
+    if (p.pipe && p.bm == 256) { fn = (const void*)attn_fwd_d128_pipe_kernel<T, SPARSE, 8>; slot = 2; }
+    else if (p.pipe) { fn = (const void*)attn_fwd_d128_pipe_kernel<T, SPARSE, 4>; slot = 1; }
+    else { fn = (const void*)attn_fwd_d128_kernel<T, SPARSE>; slot = 0; }
   } else {
     fn = (const void*)attn_fwd_kernel<T, D, SPARSE>;
     smem = Smem<D>::BYTES;
+    slot = 0;
   }
-  static bool attr_done[2] = {false, false};  // benign race: the call is idempotent
-  if (!attr_done[pipe]) {
+  static bool attr_done[3] = {false, false, false};  // benign race: the call is idempotent
+  if (!attr_done[slot]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_done[pipe] = true;
+    attr_done[slot] = true;
   }
   if constexpr (D == 128) {
-    if (pipe)
-      hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+    if (slot == 2)
+      hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, SPARSE, 8>), dim3((unsigned)nblocks), dim3(512), smem, stream, p);
+    else if (slot == 1)
+      hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, SPARSE, 4>), dim3((unsigned)nblocks), dim3(256), smem, stream, p);
     else
       hipLaunchKernelGGL((attn_fwd_d128_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
   } else {
@@ -1243,6 +1253,27 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
   }
   PA_CHECK_LAUNCH("attention kernel");
   return PA_OK;
+}
+
+// Picks the kernel and the query rows per workgroup.  The pipelined head_dim-128 kernel needs K and
+// V to span less than 4 GiB (32-bit buffer offsets).  128 rows = 4 wavefronts, two workgroups per
+// CU (the default); 256 rows = 8 wavefronts sharing one K/V stream (half the tile copies per flop),
+// selectable with PARAATTN_BM=256 where block-sparse query blocks allow it.
+static int choose_bm(AttnParams& p, int D, int q_block) {
+  p.pipe = 0;
+  if (D != 128) return 128;
+  if (p.Skv <= 0 || (uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB ||
+      (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB)
+    return 128;
+  p.pipe = 1;
+  const int B = p.B, H = p.H, Sq = p.Sq;
+  const char* force = getenv("PARAATTN_BM");  // tuning aid: 128 or 256
+  if (force && (atoi(force) == 128 || atoi(force) == 256)) {
+    if (atoi(force) == 256 && q_block % 256) return 128;
+    return atoi(force);
+  }
+  (void)B; (void)H; (void)Sq;
+  return 128;  // measured equal to 256 at the 119k-token shape (63.5 % vs 60.3 % MFMA busy, higher clock at 256)
 }
 
 template <bool SPARSE>
@@ -1266,7 +1297,8 @@ extern "C" int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void
   AttnParams p;
   fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
   p.kv_len = kv_len;
-  p.n_qtiles = (Sq + BM - 1) / BM;
+  p.bm = choose_bm(p, D, 256);
+  p.n_qtiles = (Sq + p.bm - 1) / p.bm;
   return dispatch_attn<false>(p, dtype, D, (hipStream_t)stream);
 }
 
@@ -1315,10 +1347,11 @@ extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void*
   p.runs = runs_ws;
   p.Hm = Hm; p.nQ = nQ; p.cap = nK / 2 + 3;
   p.q_lo = q_lo; p.q_block = q_block;
-  p.tiles_left = (q_lo + BM - 1) / BM;
-  p.tiles_per_block = (q_block + BM - 1) / BM;
+  p.bm = choose_bm(p, D, (q_block % 256 == 0 && q_lo % 256 == 0) ? 256 : 128);
+  p.tiles_left = (q_lo + p.bm - 1) / p.bm;
+  p.tiles_per_block = (q_block + p.bm - 1) / p.bm;
   const int q_hi = q_lo + nQ * q_block;
-  const int tiles_right = (Sq - q_hi + BM - 1) / BM;
+  const int tiles_right = (Sq - q_hi + p.bm - 1) / p.bm;
   p.n_qtiles = p.tiles_left + nQ * p.tiles_per_block + tiles_right;
   return dispatch_attn<true>(p, dtype, D, (hipStream_t)stream);
 }
