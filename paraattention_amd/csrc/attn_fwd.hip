@@ -1265,6 +1265,8 @@ static int choose_bm(AttnParams& p, int D, int q_block) {
   if (p.Skv <= 0 || (uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB ||
       (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB)
     return 128;
+  const char* nopipe = getenv("PARAATTN_NO_PIPE");  // test aid: exercise the kernel without offset limits
+  if (nopipe && nopipe[0] == '1') return 128;
   p.pipe = 1;
   const int B = p.B, H = p.H, Sq = p.Sq;
   const char* force = getenv("PARAATTN_BM");  // tuning aid: 128 or 256

@@ -158,6 +158,24 @@ def test_key_mask_and_sparse_kv(cuda):
         _check(out, lse, ref_out, ref_lse, "key mask")
 
 
+@pytest.mark.parametrize("env", [{"PARAATTN_NO_PIPE": "1"}, {"PARAATTN_BM": "256"}])
+def test_alternative_kernels(cuda, env, monkeypatch):
+    """The head_dim-128 kernel without 32-bit offset limits (taken when K or V spans 4 GiB or more) and the
+    8-wavefront workgroup variant compute the same thing as the default kernel."""
+    import os
+
+    cases = [(1, 2, 300, 434), (2, 1, 129, 1000), (1, 1, 64, 64), (1, 3, 1000, 77)]
+    for B, H, Sq, Skv in cases:
+        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=Sq + Skv)
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+        for name, val in env.items():
+            monkeypatch.setenv(name, val)
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
+        for name in env:
+            monkeypatch.delenv(name)
+        _check(out, lse, ref_out, ref_lse, f"{env} {(B, H, Sq, Skv)}")
+
+
 def test_unsupported_raise(cuda):
     q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 128))
     with pytest.raises(NotImplementedError):
