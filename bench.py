@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM-side traffic per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two rocprofv3 --pmc
 # runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy; profiles/kernels_bench_workloads.md)
-TRAFFIC = {"attn": 6.528e9, "merge": 4.634e8, "fbcache": 6.710e8, "sparse": 2.132e10}
+TRAFFIC = {"attn": 6.988e9, "merge": 4.629e8, "fbcache": 6.710e8, "sparse": 2.135e10}
 
 
 def _time_calls(fn, steps, warmup):

@@ -731,6 +731,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
     if (!have) break;
     tile_step(std::integral_constant<int, 1>{});
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the wavefront ends
 
   // ---- epilogue -----------------------------------------------------------------------------------
   float l_tot;
@@ -1065,6 +1066,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     if (!have) break;
     tile_step(std::integral_constant<int, 1>{});
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the wavefront ends
 
   // ---- epilogue -----------------------------------------------------------------------------------
   float l_tot;
