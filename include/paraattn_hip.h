@@ -69,6 +69,33 @@ PA_API int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* ou
                     float scale, const int32_t* kv_len, void* stream);
 
 /*
+ * pa_attn_fwd_lse with a workspace lent by the caller.  The reference's op
+ * (src/para_attn/ops/__init__.py:112-157) ends in an aten kernel that takes its
+ * scratch from torch's allocator; this library allocates nothing, so the caller
+ * brings it.  With a workspace of at least pa_attn_fwd_workspace_bytes() bytes
+ * (device memory, 16-byte aligned, contents irrelevant before and after) the
+ * head_dim-128 kernel may compute the query tiles of the last, partly filled
+ * round of workgroups in several key shares and fold them with the same
+ * log-sum-exp merge as pa_merge_lse, which removes the idle tail of the launch.
+ * A null or short workspace is not an error: the call then runs as
+ * pa_attn_fwd_lse does.  Results are the same to rounding.  Calls that share a
+ * workspace must not overlap.
+ */
+PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void* out, float* lse,
+                       int dtype, int B, int H, int Sq, int Skv, int D,
+                       const int64_t q_strides[3], const int64_t k_strides[3],
+                       const int64_t v_strides[3], const int64_t out_strides[3],
+                       float scale, const int32_t* kv_len, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
+ * Bytes of workspace pa_attn_fwd_lse_ws can use for this problem on the current
+ * device (0: it would not split).  Depends on the device's CU count.
+ */
+PA_API size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
+                                   const int64_t k_strides[3], const int64_t v_strides[3]);
+
+/*
  * Block-sparse attention forward: query block i (of q_block rows, counted from
  * q_lo) attends key block j (of kv_block rows, counted from kv_lo) iff
  * block_mask[hm,i,j] != 0; query rows outside [q_lo, q_lo + nQ*q_block) attend

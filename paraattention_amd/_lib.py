@@ -39,6 +39,12 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _vp],
     ),
+    "pa_attn_fwd_lse_ws": (
+        _i,
+        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp,
+         _vp, _sz, _vp],
+    ),
+    "pa_attn_fwd_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _strides, _strides]),
     "pa_attn_fwd_blocksparse": (
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f,

@@ -23,6 +23,7 @@
 // mode (src/para_attn/sparse_attn.py:209-240).
 
 #include <stdlib.h>
+#include <string.h>
 
 #include <type_traits>
 
@@ -60,6 +61,13 @@ struct AttnParams {
   int Hm, nQ, cap;
   int q_lo, q_block;
   int tiles_left, tiles_per_block;
+  // dense pipelined kernel only: key-split tail.  Workgroups below split_main own a whole query
+  // tile; the last split_tiles query tiles are computed by split_s workgroups each, over
+  // consecutive shares of the key tiles, which leave normalised fp32 partial outputs and their
+  // LSE in the workspace (piece-major) for attn_split_merge_kernel.  split_s <= 1: no split.
+  int split_main, split_tiles, split_s;
+  float* ws_out;  // [split_s * split_tiles][bm][128]
+  float* ws_lse;  // [split_s * split_tiles][bm]
 };
 
 template <int D>
@@ -86,6 +94,13 @@ struct TileIter {
     ri = 0;
     pos = 0;
     end = len;
+  }
+  __device__ __forceinline__ void init_range(int b, int e) {
+    ranges = nullptr;
+    nranges = e > b ? 1 : 0;
+    ri = 0;
+    pos = b;
+    end = e;
   }
   __device__ __forceinline__ void init_list(const int32_t* r, int n) {
     ranges = r;
@@ -792,13 +807,30 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   const int l32 = lane & 31;
   const int hh = lane >> 5;
 
-  const int qt = blockIdx.x % p.n_qtiles;
-  const int bh = blockIdx.x / p.n_qtiles;
+  int tile = blockIdx.x;
+  int piece_slot = -1;  // >= 0: this workgroup computes one key share of a split query tile
+  if constexpr (!SPARSE) {
+    if (p.split_s > 1 && tile >= p.split_main) {
+      piece_slot = tile - p.split_main;
+      tile = p.split_main + piece_slot % p.split_tiles;
+    }
+  }
+  const int qt = tile % p.n_qtiles;
+  const int bh = tile / p.n_qtiles;
   const int head = bh % p.H;
   const int batch = bh / p.H;
   int row_begin, row_end;
   TileIter it;
   decode_block<SPARSE>(p, qt, head, batch, row_begin, row_end, it);
+  if constexpr (!SPARSE) {
+    if (piece_slot >= 0) {
+      const int len = it.end;
+      const int nkt = (len + BN - 1) / BN;
+      const int piece = piece_slot / p.split_tiles;
+      const int t0 = (int)((int64_t)piece * nkt / p.split_s), t1 = (int)((int64_t)(piece + 1) * nkt / p.split_s);
+      it.init_range(t0 * BN, t1 * BN < len ? t1 * BN : len);
+    }
+  }
 
   const uint16_t* qbase = (const uint16_t*)p.q + batch * p.qs_b + head * p.qs_h;
   const char* kbytes = (const char*)((const uint16_t*)p.k + batch * p.ks_b + head * p.ks_h);
@@ -845,12 +877,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   constexpr uint32_t OOB = PIPE_OOB;  // first key of a tile that does not exist; also its soffset
   // i-th of the four copy instructions of the K (V) tile starting at key n0, into buffer `buf`
   auto dma_k1 = [&](int buf, uint32_t n0, int i) {
-    const uint32_t soff = n0 == OOB ? OOB : (n0 + RS * i) * ks_bytes;
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * ks_bytes);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_k + buf * TILE_BYTES + i * (RS * 256)), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
   };
   auto dma_v1 = [&](int buf, uint32_t n0, int i) {
-    const uint32_t soff = n0 == OOB ? OOB : (n0 + RS * i) * vs_bytes;
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * vs_bytes);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_v + buf * TILE_BYTES + i * (RS * 256)), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
   };
@@ -1075,6 +1107,23 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
   }
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  if constexpr (!SPARSE) {
+    if (piece_slot >= 0) {  // partial result of one key share: fp32, into the workspace
+      if (row_ok) {
+        const int64_t wrow = (int64_t)piece_slot * p.bm + (my_row - row_begin);
+        float* wp = p.ws_out + wrow * 128;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            float4 w = {o[db][4 * a] * inv, o[db][4 * a + 1] * inv, o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv};
+            *(float4*)(wp + 32 * db + 8 * a + 4 * hh) = w;
+          }
+        if (hh == 0) p.ws_lse[wrow] = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      }
+      return;
+    }
+  }
   if (row_ok) {
     uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)my_row * p.os_s;
 #pragma unroll
@@ -1091,6 +1140,45 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       p.lse[((int64_t)batch * p.H + head) * p.Sq + my_row] = lse;
     }
   }
+}
+
+// Folds the split_s partial results of each split query tile into out and lse: the log-sum-exp
+// merge of torch's _SDPAMerger (used by src/para_attn/sparse_attn.py:174-189) over all pieces at
+// once.  One thread = 8 consecutive output elements of one query row; 16 rows per workgroup.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_split_merge_kernel(const AttnParams p) {
+  const int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int c8 = (threadIdx.x & 15) * 8;
+  const int tl = (int)(r / p.bm), local = (int)(r % p.bm);
+  if (tl >= p.split_tiles) return;
+  const int tile = p.split_main + tl;
+  const int qt = tile % p.n_qtiles, bh = tile / p.n_qtiles;
+  const int head = bh % p.H, batch = bh / p.H;
+  const int qrow = qt * p.bm + local;
+  if (qrow >= p.Sq) return;
+  float m = -INFINITY;
+  for (int i = 0; i < p.split_s; ++i) m = fmaxf(m, p.ws_lse[((int64_t)i * p.split_tiles + tl) * p.bm + local]);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+  if (m > -INFINITY) {
+    for (int i = 0; i < p.split_s; ++i) {
+      const int64_t wrow = ((int64_t)i * p.split_tiles + tl) * p.bm + local;
+      const float w = __expf(p.ws_lse[wrow] - m);  // an empty share has LSE -inf: weight 0
+      const float4 a = *(const float4*)(p.ws_out + wrow * 128 + c8);
+      const float4 b = *(const float4*)(p.ws_out + wrow * 128 + c8 + 4);
+      den += w;
+      acc[0] += w * a.x; acc[1] += w * a.y; acc[2] += w * a.z; acc[3] += w * a.w;
+      acc[4] += w * b.x; acc[5] += w * b.y; acc[6] += w * b.z; acc[7] += w * b.w;
+    }
+  }
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  u32x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = T::pack2(acc[2 * i] * inv, acc[2 * i + 1] * inv);
+  uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)qrow * p.os_s + c8;
+  *(u32x4*)op = w;
+  if (p.lse != nullptr && c8 == 0)
+    p.lse[((int64_t)batch * p.H + head) * p.Sq + qrow] = den > 0.f ? m + __logf(den) : -INFINITY;
 }
 
 // Turns a [Hm,nQ,nK] block mask into per-segment lists of key ranges.
@@ -1218,12 +1306,14 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.runs = nullptr;
   p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.tiles_left = 0; p.tiles_per_block = 0;
   p.bm = BM; p.pipe = 0;
+  p.split_main = 0; p.split_tiles = 0; p.split_s = 0; p.ws_out = nullptr; p.ws_lse = nullptr;
 }
 
 template <typename T, int D, bool SPARSE>
 static int launch_attn(const AttnParams& p, hipStream_t stream) {
-  const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
+  int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
   if (nblocks == 0) return PA_OK;
+  if (p.split_s > 1) nblocks = (int64_t)p.split_main + (int64_t)p.split_tiles * p.split_s;
   const void* fn;
   size_t smem;
   int slot;
@@ -1254,30 +1344,123 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     hipLaunchKernelGGL((attn_fwd_kernel<T, D, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
   }
   PA_CHECK_LAUNCH("attention kernel");
+  if constexpr (D == 128 && !SPARSE) {
+    if (p.split_s > 1) {
+      const int64_t rows = (int64_t)p.split_tiles * p.bm;
+      hipLaunchKernelGGL((attn_split_merge_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream, p);
+      PA_CHECK_LAUNCH("attention split merge kernel");
+    }
+  }
   return PA_OK;
 }
 
-// Picks the kernel and the query rows per workgroup.  The pipelined head_dim-128 kernel needs K and
-// V to span less than 4 GiB (32-bit buffer offsets).  128 rows = 4 wavefronts, two workgroups per
-// CU (the default); 256 rows = 8 wavefronts sharing one K/V stream (half the tile copies per flop),
-// selectable with PARAATTN_BM=256 where block-sparse query blocks allow it.
-static int choose_bm(AttnParams& p, int D, int q_block) {
+// Compute units of the current device (0 if it cannot be asked), cached per device.
+static int device_cus() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cus[dev] = n;  // benign race: every thread writes the same value
+  }
+  return cus[dev];
+}
+
+// Key-split tail.  All workgroups of the dense kernel cost the same, so a grid of n_tiles
+// workgroups on `slots` resident places takes ceil(n_tiles / slots) rounds however empty the last
+// round is.  Computing the last T query tiles in s key shares each (T*s workgroups of 1/s the
+// length, plus a small merge) turns that into (n_tiles - T) / slots + ceil(T*s / slots) / s.
+// T is the remainder of n_tiles modulo slots, or that plus one more round; s <= 8 and every share
+// keeps at least 16 key tiles.  A workgroup's fixed cost (Q load, first tile copies, output) is
+// priced at 4 key tiles, so a share of a tile with n key tiles costs (n/s + 4) / (n + 4) of a
+// whole one.  Returns s = 1 unless the estimate improves by 3 %.
+struct SplitPlan {
+  int tiles, s;
+  double rounds;
+};
+static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, bool allow) {
+  if (slots <= 0) return {0, 1, 1.0};  // no device to ask: no estimate, no split
+  SplitPlan best = {0, 1, (double)((n_tiles + slots - 1) / slots)};
+  if (!allow || n_tiles % slots == 0) return best;
+  SplitPlan found = best;
+  double best_found = best.rounds;
+  for (int extra = 0; extra < 2; ++extra) {
+    const int64_t T = n_tiles % slots + (int64_t)extra * slots;
+    if (T > n_tiles || T * 8 > 0x7fffffffLL) break;
+    for (int s = 2; s <= 8 && kv_tiles / s >= 16; ++s) {
+      const double share = ((double)kv_tiles / s + 4.0) / ((double)kv_tiles + 4.0);
+      const double r = (double)((n_tiles - T) / slots) + (double)((T * s + slots - 1) / slots) * share + 0.02;
+      if (r < best.rounds * 0.97 && r < best_found) { best_found = r; found = {(int)T, s, r}; }
+    }
+  }
+  return found;
+}
+
+static bool env_is(const char* name, const char* val) {
+  const char* e = getenv(name);
+  return e && strcmp(e, val) == 0;
+}
+
+// Bytes of workspace the key-split tail of the plan for bm rows per workgroup needs.
+static size_t split_ws_bytes(const SplitPlan& pl, int bm) {
+  return pl.s > 1 ? (size_t)pl.tiles * pl.s * bm * (128 + 1) * sizeof(float) : 0;
+}
+
+// Picks the kernel, the query rows per workgroup and the key-split tail.  The pipelined
+// head_dim-128 kernel needs K and V to span less than 4 GiB (32-bit buffer offsets).  128 rows = 4
+// wavefronts, two workgroups per CU; 256 rows = 8 wavefronts sharing one K/V stream (half the tile
+// copies per flop: measured 5.5 % more throughput per full round at the 119k-token shape, but one
+// workgroup per CU makes a partly filled last round dearer).  The choice is the smaller estimate
+// of rounds / throughput; PARAATTN_BM=128|256 forces it, PARAATTN_NO_SPLIT=1 forbids the split.
+// `ws_bytes` is what the caller can lend (0: none); q_block limits 256 for block-sparse launches.
+static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t ws_bytes, size_t* ws_needed) {
+  if (ws_needed) *ws_needed = 0;
   p.pipe = 0;
-  if (D != 128) return 128;
+  p.bm = 128;
+  p.split_s = 0;
+  auto finish = [&] { p.n_qtiles = (p.Sq + p.bm - 1) / p.bm; };
+  if (D != 128) return finish();
   if (p.Skv <= 0 || (uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB ||
       (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB)
-    return 128;
-  const char* nopipe = getenv("PARAATTN_NO_PIPE");  // test aid: exercise the kernel without offset limits
-  if (nopipe && nopipe[0] == '1') return 128;
+    return finish();
+  if (env_is("PARAATTN_NO_PIPE", "1")) return finish();  // test aid: the kernel without offset limits
   p.pipe = 1;
-  const int B = p.B, H = p.H, Sq = p.Sq;
-  const char* force = getenv("PARAATTN_BM");  // tuning aid: 128 or 256
-  if (force && (atoi(force) == 128 || atoi(force) == 256)) {
-    if (atoi(force) == 256 && q_block % 256) return 128;
-    return atoi(force);
+  const char* force = getenv("PARAATTN_BM");  // tuning aid
+  const int forced = force ? atoi(force) : 0;
+  if (!dense) {  // block-sparse: workgroups differ in length, no split
+    if (forced == 256 && q_block % 256 == 0) p.bm = 256;
+    return finish();
   }
-  (void)B; (void)H; (void)Sq;
-  return 128;  // measured equal to 256 at the 119k-token shape (63.5 % vs 60.3 % MFMA busy, higher clock at 256)
+  const int cus = device_cus();
+  const bool allow = cus > 0 && !env_is("PARAATTN_NO_SPLIT", "1") && (ws_needed != nullptr || ws_bytes > 0);
+  const int kv_tiles = (p.Skv + BN - 1) / BN;
+  const int64_t bh = (int64_t)p.B * p.H;
+  const int64_t n128 = bh * ((p.Sq + 127) / 128), n256 = bh * ((p.Sq + 255) / 256);
+  SplitPlan p128 = plan_split(n128, 2 * cus, kv_tiles, allow), p256 = plan_split(n256, cus, kv_tiles, allow);
+  if (!ws_needed) {  // the plan must fit what was lent
+    if (split_ws_bytes(p128, 128) > ws_bytes) p128 = plan_split(n128, 2 * cus, kv_tiles, false);
+    if (split_ws_bytes(p256, 256) > ws_bytes) p256 = plan_split(n256, cus, kv_tiles, false);
+  }
+  // an unsplit last round of 128-row workgroups that leaves every CU at most one of them runs
+  // about 1.5 times faster per workgroup
+  double r128 = p128.rounds, r256 = p256.rounds;
+  if (cus > 0 && p128.s == 1 && n128 % (2 * cus) != 0 && n128 % (2 * cus) <= cus) r128 -= 0.33;
+  // measured throughput of a full round of 256-row workgroups against one of 128-row workgroups:
+  // +4..10 % from 4608 keys up, -4 % at 512 keys
+  const double gain256 = kv_tiles >= 32 ? 1.055 : 0.95;
+  bool use256 = cus > 0 && n256 >= cus && r256 / gain256 < r128;
+  if (forced == 128) use256 = false;
+  if (forced == 256) use256 = true;
+  const SplitPlan& pl = use256 ? p256 : p128;
+  p.bm = use256 ? 256 : 128;
+  finish();
+  if (ws_needed) *ws_needed = split_ws_bytes(pl, p.bm);
+  if (pl.s > 1 && !ws_needed) {
+    p.split_s = pl.s;
+    p.split_tiles = pl.tiles;
+    p.split_main = (int)(bh * p.n_qtiles - pl.tiles);
+  }
 }
 
 template <bool SPARSE>
@@ -1290,20 +1473,54 @@ static int dispatch_attn(const AttnParams& p, int dtype, int D, hipStream_t stre
   return launch_attn<F16, 64, SPARSE>(p, stream);
 }
 
+static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out, float* lse,
+                          int dtype, int B, int H, int Sq, int Skv, int D,
+                          const int64_t q_strides[3], const int64_t k_strides[3],
+                          const int64_t v_strides[3], const int64_t out_strides[3], float scale,
+                          const int32_t* kv_len, void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                        out_strides, scale);
+  if (rc) return rc;
+  if (workspace && ((uintptr_t)workspace) % 16) PA_FAIL(PA_ERR_WORKSPACE, "attention workspace not 16-byte aligned");
+  AttnParams p;
+  fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
+  p.kv_len = kv_len;
+  choose_kernel(p, D, 256, true, workspace ? workspace_bytes : 0, nullptr);
+  if (p.split_s > 1) {
+    p.ws_out = (float*)workspace;
+    p.ws_lse = p.ws_out + (size_t)p.split_tiles * p.split_s * p.bm * 128;
+  }
+  return dispatch_attn<false>(p, dtype, D, (hipStream_t)stream);
+}
+
 extern "C" int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* out, float* lse,
                                int dtype, int B, int H, int Sq, int Skv, int D,
                                const int64_t q_strides[3], const int64_t k_strides[3],
                                const int64_t v_strides[3], const int64_t out_strides[3],
                                float scale, const int32_t* kv_len, void* stream) {
-  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
-                        out_strides, scale);
-  if (rc) return rc;
+  return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                        out_strides, scale, kv_len, nullptr, 0, stream);
+}
+
+extern "C" int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void* out, float* lse,
+                                  int dtype, int B, int H, int Sq, int Skv, int D,
+                                  const int64_t q_strides[3], const int64_t k_strides[3],
+                                  const int64_t v_strides[3], const int64_t out_strides[3],
+                                  float scale, const int32_t* kv_len, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                        out_strides, scale, kv_len, workspace, workspace_bytes, stream);
+}
+
+extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
+                                              const int64_t k_strides[3], const int64_t v_strides[3]) {
+  if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D != 128 || !k_strides || !v_strides) return 0;
   AttnParams p;
-  fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
-  p.kv_len = kv_len;
-  p.bm = choose_bm(p, D, 256);
-  p.n_qtiles = (Sq + p.bm - 1) / p.bm;
-  return dispatch_attn<false>(p, dtype, D, (hipStream_t)stream);
+  const int64_t zero[3] = {0, 0, 0};
+  fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
+  size_t need = 0;
+  choose_kernel(p, D, 256, true, 0, &need);
+  return need;
 }
 
 extern "C" size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK) {
@@ -1351,7 +1568,7 @@ extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void*
   p.runs = runs_ws;
   p.Hm = Hm; p.nQ = nQ; p.cap = nK / 2 + 3;
   p.q_lo = q_lo; p.q_block = q_block;
-  p.bm = choose_bm(p, D, (q_block % 256 == 0 && q_lo % 256 == 0) ? 256 : 128);
+  choose_kernel(p, D, (q_block % 256 == 0 && q_lo % 256 == 0) ? 256 : 128, false, 0, nullptr);
   p.tiles_left = (q_lo + p.bm - 1) / p.bm;
   p.tiles_per_block = (q_block + p.bm - 1) / p.bm;
   const int q_hi = q_lo + nQ * q_block;

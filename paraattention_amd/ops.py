@@ -95,12 +95,17 @@ def _dense_forward(query, key, value, scale, want_lse, kv_len=None):
         scale = 1.0 / math.sqrt(D)
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        rc = lib.pa_attn_fwd_lse(
+        # scratch for the key-split tail of the launch (torch's caching allocator: no hipMalloc in
+        # the steady state); its lifetime on the launch stream is the allocator's business
+        ks, vs = _lib.strides3(k), _lib.strides3(v)
+        ws_bytes = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, ks, vs)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+        rc = lib.pa_attn_fwd_lse_ws(
             _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
-            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
-            float(scale), _ptr(kv_len), _stream_ptr(q.device),
+            _lib.strides3(q), ks, vs, _lib.strides3(out),
+            float(scale), _ptr(kv_len), _ptr(ws), ws_bytes, _stream_ptr(q.device),
         )
-    _lib.check(rc, "pa_attn_fwd_lse")
+    _lib.check(rc, "pa_attn_fwd_lse_ws")
     return out, lse
 
 

@@ -176,6 +176,61 @@ def test_alternative_kernels(cuda, env, monkeypatch):
         _check(out, lse, ref_out, ref_lse, f"{env} {(B, H, Sq, Skv)}")
 
 
+@pytest.mark.parametrize("bm", ["128", "256"])
+def test_key_split_tail(cuda, bm, monkeypatch):
+    """Grids a little over a whole number of rounds: the query tiles of the last round are computed in key
+    shares (fp32 partials in a workspace) and merged.  Checked against the oracle, against the unsplit launch,
+    with per-batch key counts that leave some shares empty, and with a strided output."""
+    from paraattention_amd import _lib
+
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rows = int(bm)
+    slots = cus * (2 if bm == "128" else 1)
+    B, H, D = 2, 4, 128
+    tiles_per_head = slots // (B * H) + 5   # 40 tiles over a whole round
+    Sq = tiles_per_head * rows - 19          # ragged last tile
+    Skv = 64 * 40 + 37
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=77)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    monkeypatch.setenv("PARAATTN_BM", bm)
+    need = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, _lib.strides3(kd), _lib.strides3(vd))
+    assert need > 0, "this shape is meant to take the key-split path"
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q, k, v)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd)
+    _check(out, lse, ref_out.float().numpy(), ref_lse.numpy(), f"split bm={bm}")
+    monkeypatch.setenv("PARAATTN_NO_SPLIT", "1")
+    assert lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, _lib.strides3(kd), _lib.strides3(vd)) == 0
+    out1, lse1 = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd)
+    monkeypatch.delenv("PARAATTN_NO_SPLIT")
+    assert (out.float() - out1.float()).abs().max().item() <= 2e-2
+    assert (lse - lse1).abs().max().item() <= 1e-4
+    # a workspace that is too short is not an error: the launch is the unsplit one
+    import ctypes
+
+    out3, lse3 = torch.empty_like(out), torch.empty_like(lse)
+    short = torch.empty(64, dtype=torch.uint8, device=cuda)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    rc = lib.pa_attn_fwd_lse_ws(vp(qd), vp(kd), vp(vd), vp(out3), vp(lse3), 0, B, H, Sq, Skv, D, _lib.strides3(qd),
+                                _lib.strides3(kd), _lib.strides3(vd), _lib.strides3(out3), 1.0 / math.sqrt(D), None,
+                                vp(short), short.numel(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out3, out1) and torch.equal(lse3, lse1)
+    # per-batch key counts: batch 1 keeps 40 keys, so all but one of its shares are empty
+    lens = torch.tensor([Skv - 3, 40])
+    keep = torch.arange(Skv)[None, :] < lens[:, None]
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :1, -300:].float().numpy(), k[:, :1].float().numpy(), v[:, :1].float().numpy(),
+                                          None, keep[:, None, None, :].numpy())
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, keep[:, None, None, :].to(cuda))
+    _check(out[:, :1, -300:], lse[:, :1, -300:], ref_out, ref_lse, f"split bm={bm} key counts")
+    # [B,S,H,D] memory for q and the output
+    qs = qd.transpose(1, 2).contiguous().transpose(1, 2)
+    out2, lse2 = torch.ops.para_attn.attention_forward_with_lse(qs, kd, vd, keep[:, None, None, :].to(cuda))
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+    monkeypatch.delenv("PARAATTN_BM")
+
+
 def test_unsupported_raise(cuda):
     q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 128))
     with pytest.raises(NotImplementedError):
