@@ -2,7 +2,7 @@
 (B=1, 3 of 24 heads, S=119056, D=128, bf16, q/k RMS-normalised), one MI355X.
 
 Prints ONE JSON line.  ``value`` is attention TFLOP/s (4*B*H*Sq*Skv*D flop per call) with inputs
-resident in HBM; ``roofline`` prices the attention kernel against the bf16 dense MFMA peak;
+resident in HBM (a call = the attention kernel plus the 8 us merge of its key-split tail); ``roofline`` prices the attention kernel against the bf16 dense MFMA peak;
 ``cpu_baseline`` is torch's CPU SDPA (the library routine the reference's SDPA path is checked
 against) on a bounded sample of the same workload; ``extras`` holds the bandwidth-bound kernels
 (ring merge step, FBCache reduction) against the HBM peak and the block-sparse mode.
@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM-side traffic per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two rocprofv3 --pmc
 # runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy; profiles/kernels_bench_workloads.md)
-TRAFFIC = {"attn": 6.988e9, "merge": 4.629e8, "fbcache": 6.710e8, "sparse": 2.135e10}
+TRAFFIC = {"attn": 4.164e9, "merge": 4.631e8, "fbcache": 6.710e8, "sparse": 2.031e10}
 
 
 def _time_calls(fn, steps, warmup):

@@ -65,6 +65,7 @@ struct AttnParams {
   // tile; the last split_tiles query tiles are computed by split_s workgroups each, over
   // consecutive shares of the key tiles, which leave normalised fp32 partial outputs and their
   // LSE in the workspace (piece-major) for attn_split_merge_kernel.  split_s <= 1: no split.
+  int xcd_chunk;  // block-sparse pipelined kernel: ceil(workgroups / 8), 0 = plain order
   int split_main, split_tiles, split_s;
   float* ws_out;  // [split_s * split_tiles][bm][128]
   float* ws_lse;  // [split_s * split_tiles][bm]
@@ -809,6 +810,15 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
 
   int tile = blockIdx.x;
   int piece_slot = -1;  // >= 0: this workgroup computes one key share of a split query tile
+  if constexpr (SPARSE) {
+    // Workgroups go to the 8 XCDs in turn.  Give each XCD a contiguous eighth of the (head, query
+    // tile) list, so that the workgroups sharing an L2 work on neighbouring query blocks of one
+    // head, whose kept key blocks overlap, instead of every eighth block of several heads.
+    if (p.xcd_chunk > 0) {
+      tile = (tile & 7) * p.xcd_chunk + (tile >> 3);
+      if (tile >= p.B * p.H * p.n_qtiles) return;
+    }
+  }
   if constexpr (!SPARSE) {
     if (p.split_s > 1 && tile >= p.split_main) {
       piece_slot = tile - p.split_main;
@@ -1306,6 +1316,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.runs = nullptr;
   p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.tiles_left = 0; p.tiles_per_block = 0;
   p.bm = BM; p.pipe = 0;
+  p.xcd_chunk = 0;
   p.split_main = 0; p.split_tiles = 0; p.split_s = 0; p.ws_out = nullptr; p.ws_lse = nullptr;
 }
 
@@ -1314,6 +1325,7 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
   int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
   if (nblocks == 0) return PA_OK;
   if (p.split_s > 1) nblocks = (int64_t)p.split_main + (int64_t)p.split_tiles * p.split_s;
+  if (p.xcd_chunk > 0) nblocks = 8 * (int64_t)p.xcd_chunk;
   const void* fn;
   size_t smem;
   int slot;
@@ -1574,5 +1586,7 @@ extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void*
   const int q_hi = q_lo + nQ * q_block;
   const int tiles_right = (Sq - q_hi + p.bm - 1) / p.bm;
   p.n_qtiles = p.tiles_left + nQ * p.tiles_per_block + tiles_right;
+  if (D == 128 && p.pipe && !env_is("PARAATTN_NO_XCD_ORDER", "1"))
+    p.xcd_chunk = (int)(((int64_t)B * H * p.n_qtiles + 7) / 8);
   return dispatch_attn<true>(p, dtype, D, (hipStream_t)stream);
 }
