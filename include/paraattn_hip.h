@@ -89,7 +89,32 @@ PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void*
                        size_t workspace_bytes, void* stream);
 
 /*
- * Bytes of workspace pa_attn_fwd_lse_ws can use for this problem on the current
+ * One step of a same-GPU ring sweep in one launch: attention of q against one
+ * key/value block, folded into the running pair (acc_out, acc_lse) by the
+ * log-sum-exp merge of pa_merge_lse inside the attention kernel's epilogue.
+ * Replaces, per step of torch's _templated_ring_attention loop as the reference
+ * drives it (src/para_attn/para_attn_interface.py:164-197), the attention op
+ * (src/para_attn/ops/__init__.py:112-157) plus _SDPAMerger.step: the block's
+ * own 16-bit output and the merge pass over it never exist.
+ *
+ * acc_out: fp32 [B,H,Sq,D] contiguous; acc_lse: fp32 [B,H,Sq]; both updated in
+ * place.  first != 0: the pair holds nothing yet and is not read (no need to
+ * initialise it).  out == NULL: acc_out receives the folded output.  out != NULL
+ * (the last step): the folded output is written to out in `dtype` with
+ * out_strides, acc_out is left as it was, acc_lse is the final LSE.
+ * workspace: as for pa_attn_fwd_lse_ws (may be NULL).  head_dim 128 with K and
+ * V below 4 GiB per (batch, head) only; otherwise PA_ERR_UNSUPPORTED (run
+ * pa_attn_fwd_lse and pa_merge_lse instead).
+ */
+PA_API int pa_attn_fwd_accumulate(const void* q, const void* k, const void* v, float* acc_out,
+                           float* acc_lse, void* out, int dtype, int B, int H, int Sq, int Skv,
+                           int D, const int64_t q_strides[3], const int64_t k_strides[3],
+                           const int64_t v_strides[3], const int64_t out_strides[3], float scale,
+                           const int32_t* kv_len, int first, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/*
+ * Bytes of workspace pa_attn_fwd_lse_ws and pa_attn_fwd_accumulate can use for this problem on the current
  * device (0: it would not split).  Depends on the device's CU count.
  */
 PA_API size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,

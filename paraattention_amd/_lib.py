@@ -44,6 +44,11 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp,
          _vp, _sz, _vp],
     ),
+    "pa_attn_fwd_accumulate": (
+        _i,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp,
+         _i, _vp, _sz, _vp],
+    ),
     "pa_attn_fwd_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _strides, _strides]),
     "pa_attn_fwd_blocksparse": (
         _i,

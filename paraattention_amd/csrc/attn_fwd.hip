@@ -69,6 +69,14 @@ struct AttnParams {
   int split_main, split_tiles, split_s;
   float* ws_out;  // [split_s * split_tiles][bm][128]
   float* ws_lse;  // [split_s * split_tiles][bm]
+  // dense pipelined kernel only: ring accumulation.  With acc_out set, the result of this launch is
+  // folded into the running pair (acc_out fp32 [B,H,Sq,128] contiguous, acc_lse [B,H,Sq]) by the
+  // log-sum-exp merge instead of being stored on its own.  acc_first: the pair holds nothing yet
+  // and is not read.  With `out` also set (last step) the folded output goes to `out` in the
+  // activation type and acc_out is left alone; acc_lse is updated either way; `lse` is unused.
+  float* acc_out;
+  float* acc_lse;
+  int acc_first;
 };
 
 template <int D>
@@ -1133,6 +1141,46 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       }
       return;
     }
+    if (p.acc_out != nullptr) {  // fold into the running (out, lse) pair
+      if (row_ok) {
+        const int64_t ridx = ((int64_t)batch * p.H + head) * p.Sq + my_row;
+        const float blk = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+        const float old = p.acc_first ? -INFINITY : p.acc_lse[ridx];
+        const float mx = fmaxf(old, blk);
+        float w_old = 0.f, w_blk = 0.f, lse_new = -INFINITY;
+        if (mx > -INFINITY) {
+          const float e_old = __expf(old - mx), e_blk = __expf(blk - mx);
+          const float den = e_old + e_blk;
+          w_old = e_old / den;
+          w_blk = e_blk / den * inv;
+          lse_new = mx + __logf(den);
+        }
+        float* ap = p.acc_out + ridx * 128;
+        uint16_t* op = p.out ? (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)my_row * p.os_s : nullptr;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            const int d0 = 32 * db + 8 * a + 4 * hh;
+            float4 r = {0.f, 0.f, 0.f, 0.f};
+            if (!p.acc_first && w_old > 0.f) r = *(const float4*)(ap + d0);
+            r.x = r.x * w_old + o[db][4 * a] * w_blk;
+            r.y = r.y * w_old + o[db][4 * a + 1] * w_blk;
+            r.z = r.z * w_old + o[db][4 * a + 2] * w_blk;
+            r.w = r.w * w_old + o[db][4 * a + 3] * w_blk;
+            if (op) {
+              u32x2 w;
+              w[0] = T::pack2(r.x, r.y);
+              w[1] = T::pack2(r.z, r.w);
+              *(u32x2*)(op + d0) = w;
+            } else {
+              *(float4*)(ap + d0) = r;
+            }
+          }
+        if (hh == 0) p.acc_lse[ridx] = lse_new;
+      }
+      return;
+    }
   }
   if (row_ok) {
     uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)my_row * p.os_s;
@@ -1166,10 +1214,21 @@ __global__ __launch_bounds__(256) void attn_split_merge_kernel(const AttnParams 
   const int head = bh % p.H, batch = bh / p.H;
   const int qrow = qt * p.bm + local;
   if (qrow >= p.Sq) return;
-  float m = -INFINITY;
+  const int64_t ridx = ((int64_t)batch * p.H + head) * p.Sq + qrow;
+  // ring accumulation: the running pair is one more term of the merge
+  const float old = (p.acc_out != nullptr && !p.acc_first) ? p.acc_lse[ridx] : -INFINITY;
+  float m = old;
   for (int i = 0; i < p.split_s; ++i) m = fmaxf(m, p.ws_lse[((int64_t)i * p.split_tiles + tl) * p.bm + local]);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float den = 0.f;
+  if (old > -INFINITY) {
+    const float w = __expf(old - m);
+    const float4 a = *(const float4*)(p.acc_out + ridx * 128 + c8);
+    const float4 b = *(const float4*)(p.acc_out + ridx * 128 + c8 + 4);
+    den = w;
+    acc[0] = w * a.x; acc[1] = w * a.y; acc[2] = w * a.z; acc[3] = w * a.w;
+    acc[4] = w * b.x; acc[5] = w * b.y; acc[6] = w * b.z; acc[7] = w * b.w;
+  }
   if (m > -INFINITY) {
     for (int i = 0; i < p.split_s; ++i) {
       const int64_t wrow = ((int64_t)i * p.split_tiles + tl) * p.bm + local;
@@ -1182,13 +1241,19 @@ __global__ __launch_bounds__(256) void attn_split_merge_kernel(const AttnParams 
     }
   }
   const float inv = den > 0.f ? 1.0f / den : 0.f;
-  u32x4 w;
+  if (p.out != nullptr) {
+    u32x4 w;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = T::pack2(acc[2 * i] * inv, acc[2 * i + 1] * inv);
-  uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)qrow * p.os_s + c8;
-  *(u32x4*)op = w;
-  if (p.lse != nullptr && c8 == 0)
-    p.lse[((int64_t)batch * p.H + head) * p.Sq + qrow] = den > 0.f ? m + __logf(den) : -INFINITY;
+    for (int i = 0; i < 4; ++i) w[i] = T::pack2(acc[2 * i] * inv, acc[2 * i + 1] * inv);
+    uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)qrow * p.os_s + c8;
+    *(u32x4*)op = w;
+  } else {
+    float* ap = p.acc_out + ridx * 128 + c8;
+    *(float4*)ap = float4{acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+    *(float4*)(ap + 4) = float4{acc[4] * inv, acc[5] * inv, acc[6] * inv, acc[7] * inv};
+  }
+  float* lse_dst = p.acc_out != nullptr ? p.acc_lse : p.lse;
+  if (lse_dst != nullptr && c8 == 0) lse_dst[ridx] = den > 0.f ? m + __logf(den) : -INFINITY;
 }
 
 // Turns a [Hm,nQ,nK] block mask into per-segment lists of key ranges.
@@ -1317,6 +1382,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.tiles_left = 0; p.tiles_per_block = 0;
   p.bm = BM; p.pipe = 0;
   p.xcd_chunk = 0;
+  p.acc_out = nullptr; p.acc_lse = nullptr; p.acc_first = 0;
   p.split_main = 0; p.split_tiles = 0; p.split_s = 0; p.ws_out = nullptr; p.ws_lse = nullptr;
 }
 
@@ -1489,15 +1555,29 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
                           int dtype, int B, int H, int Sq, int Skv, int D,
                           const int64_t q_strides[3], const int64_t k_strides[3],
                           const int64_t v_strides[3], const int64_t out_strides[3], float scale,
-                          const int32_t* kv_len, void* workspace, size_t workspace_bytes, void* stream) {
-  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
-                        out_strides, scale);
+                          const int32_t* kv_len, void* workspace, size_t workspace_bytes, void* stream,
+                          float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0) {
+  const int64_t zero3[3] = {0, 0, 0};
+  const bool accumulate = acc_out != nullptr;
+  if (accumulate) {
+    if (!acc_lse) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+    if (((uintptr_t)acc_out) % 16) PA_FAIL(PA_ERR_UNSUPPORTED, "accumulator not 16-byte aligned");
+    if (!out) out_strides = zero3;
+  }
+  int rc = check_common(q, k, v, accumulate && !out ? (void*)acc_out : out, dtype, B, H, Sq, Skv, D, q_strides,
+                        k_strides, v_strides, out_strides, scale);
   if (rc) return rc;
   if (workspace && ((uintptr_t)workspace) % 16) PA_FAIL(PA_ERR_WORKSPACE, "attention workspace not 16-byte aligned");
   AttnParams p;
   fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
   p.kv_len = kv_len;
   choose_kernel(p, D, 256, true, workspace ? workspace_bytes : 0, nullptr);
+  if (accumulate) {
+    if (!p.pipe)
+      PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation needs head_dim 128 and K/V below 4 GiB per head; run pa_attn_fwd_lse and pa_merge_lse");
+    p.acc_out = acc_out; p.acc_lse = acc_lse; p.acc_first = acc_first != 0;
+    p.lse = nullptr;
+  }
   if (p.split_s > 1) {
     p.ws_out = (float*)workspace;
     p.ws_lse = p.ws_out + (size_t)p.split_tiles * p.split_s * p.bm * 128;
@@ -1522,6 +1602,19 @@ extern "C" int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, v
                                   size_t workspace_bytes, void* stream) {
   return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
                         out_strides, scale, kv_len, workspace, workspace_bytes, stream);
+}
+
+extern "C" int pa_attn_fwd_accumulate(const void* q, const void* k, const void* v, float* acc_out,
+                                      float* acc_lse, void* out, int dtype, int B, int H, int Sq,
+                                      int Skv, int D, const int64_t q_strides[3],
+                                      const int64_t k_strides[3], const int64_t v_strides[3],
+                                      const int64_t out_strides[3], float scale,
+                                      const int32_t* kv_len, int first, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+  if (!acc_out || !acc_lse) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  if (out && !out_strides) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  return attn_fwd_dense(q, k, v, out, nullptr, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                        out_strides, scale, kv_len, workspace, workspace_bytes, stream, acc_out, acc_lse, first);
 }
 
 extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,

@@ -58,17 +58,34 @@ class SDPAMerger:
         return out, self._lse.reshape(self._lse_shape)
 
 
-def ring_sweep(query, key_blocks, value_blocks, *, scale=None):
+def ring_sweep(query, key_blocks, value_blocks, *, scale=None, fused=None):
     """One rank's ring-attention pass: ``query`` against successive key/value blocks.
 
     Equals one SDPA of ``query`` over the concatenation of all blocks.  The last
     merge writes the activation dtype directly, so no separate cast pass runs.
+    ``fused`` (default: when the accumulator is fp32, head_dim is 128 and there is
+    more than one block) folds each block's result into the accumulator inside
+    the attention kernel; ``fused=False`` runs attention and merge as two launches.
     Returns (out in query.dtype, fp32 lse [B,H,Sq]).
     """
     assert len(key_blocks) == len(value_blocks) and len(key_blocks) > 0
     convert = not config.attention.allow_reduced_precision_compute
     acc_dtype = torch.float32 if convert else query.dtype
     n = len(key_blocks)
+    if fused is None:
+        fused = convert and n > 1 and query.shape[-1] == 128
+    if fused:
+        # attention and merge in one launch per block: the blocks' own outputs never exist
+        B, H, Sq, D = query.shape
+        acc_out = torch.empty((B, H, Sq, D), dtype=torch.float32, device=query.device)
+        acc_lse = torch.empty((B, H, Sq), dtype=torch.float32, device=query.device)
+        try:
+            for i, (k, v) in enumerate(zip(key_blocks[:-1], value_blocks[:-1])):
+                ops.attention_forward_accumulate_(acc_out, acc_lse, query, k, v, i == 0, scale=scale)
+            out = ops.attention_forward_accumulate_final(acc_out, acc_lse, query, key_blocks[-1], value_blocks[-1], scale=scale)
+            return out, acc_lse
+        except NotImplementedError:
+            pass  # a block the fused kernel does not take (K/V of 4 GiB per head): two launches per block below
     acc_out = acc_lse = None
     for i, (k, v) in enumerate(zip(key_blocks, value_blocks)):
         out, lse = ops.attention_forward_with_lse(query, k, v, scale=scale)

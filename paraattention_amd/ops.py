@@ -15,6 +15,7 @@ Ops with a counterpart in the reference:
 Ops the reference has no name for, because there the arithmetic is a chain of
 torch elementwise calls:
   merge_attention_lse / merge_attention_lse_   (torch _SDPAMerger._merge_one)
+  attention_forward_accumulate_ / _final       (attention + merge step in one launch)
   attention_forward_block_sparse               (sparse_attn.py:74-278)
   fbcache_residual_diff                        (first_block_cache/utils.py:228-233)
   fbcache_first_residual_diff, fbcache_apply_residual (utils.py:359, 237-259)
@@ -107,6 +108,34 @@ def _dense_forward(query, key, value, scale, want_lse, kv_len=None):
         )
     _lib.check(rc, "pa_attn_fwd_lse_ws")
     return out, lse
+
+
+def _accumulate_forward(acc_out, acc_lse, query, key, value, scale, first, final):
+    """One fused ring step (pa_attn_fwd_accumulate); returns the 16-bit output if ``final``."""
+    B, H, Sq, D = query.shape
+    Skv = key.shape[2]
+    if acc_out.dtype != torch.float32 or acc_lse.dtype != torch.float32:
+        raise ValueError("accumulators must be fp32")
+    if tuple(acc_out.shape) != (B, H, Sq, D) or tuple(acc_lse.shape) != (B, H, Sq):
+        raise ValueError("accumulator shapes must be [B,H,Sq,D] and [B,H,Sq]")
+    if not acc_out.is_contiguous() or not acc_lse.is_contiguous():
+        raise ValueError("accumulators must be contiguous")
+    q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device) if final else None
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        ks, vs = _lib.strides3(k), _lib.strides3(v)
+        ws_bytes = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, ks, vs)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+        rc = lib.pa_attn_fwd_accumulate(
+            _ptr(q), _ptr(k), _ptr(v), _ptr(acc_out), _ptr(acc_lse), _ptr(out), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
+            _lib.strides3(q), ks, vs, _lib.strides3(out) if final else None,
+            float(scale), None, 1 if first else 0, _ptr(ws), ws_bytes, _stream_ptr(q.device),
+        )
+    _lib.check(rc, "pa_attn_fwd_accumulate")
+    return out
 
 
 def _masked_forward(query, key, value, attn_mask, scale, want_lse):
@@ -298,6 +327,55 @@ def merge_attention_lse_(
 @torch.library.register_fake("para_attn::merge_attention_lse_")
 def _(acc_out, acc_lse, blk_out, blk_lse):
     return None
+
+
+@torch.library.custom_op(
+    "para_attn::attention_forward_accumulate_", mutates_args=("acc_out", "acc_lse"), device_types=("cuda",)
+)
+def attention_forward_accumulate_(
+    acc_out: torch.Tensor,
+    acc_lse: torch.Tensor,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    first: bool = False,
+    *,
+    scale: Optional[float] = None,
+) -> None:
+    """Fused ring step: SDPA of ``query`` over one key/value block, merged into the fp32 running
+    pair inside the attention kernel (what attention_forward_with_lse + _SDPAMerger.step do in
+    two passes, src/para_attn/para_attn_interface.py:164-197).  ``first``: the pair is
+    uninitialised.  head_dim 128 only (NotImplementedError otherwise)."""
+    _check_sdpa_args(query, key, value, 0.0, False)
+    _accumulate_forward(acc_out, acc_lse, query, key, value, scale, first, False)
+
+
+@torch.library.register_fake("para_attn::attention_forward_accumulate_")
+def _(acc_out, acc_lse, query, key, value, first=False, *, scale=None):
+    return None
+
+
+@torch.library.custom_op(
+    "para_attn::attention_forward_accumulate_final", mutates_args=("acc_lse",), device_types=("cuda",)
+)
+def attention_forward_accumulate_final(
+    acc_out: torch.Tensor,
+    acc_lse: torch.Tensor,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    *,
+    scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Last fused ring step: returns the merged output in query's dtype (the cast of
+    _SDPAMerger.results() folded in); ``acc_lse`` becomes the final LSE, ``acc_out`` is only read."""
+    _check_sdpa_args(query, key, value, 0.0, False)
+    return _accumulate_forward(acc_out, acc_lse, query, key, value, scale, False, True)
+
+
+@torch.library.register_fake("para_attn::attention_forward_accumulate_final")
+def _(acc_out, acc_lse, query, key, value, *, scale=None):
+    return query.new_empty(query.shape)
 
 
 # ---------------------------------------------------------------------------------

@@ -73,17 +73,60 @@ def test_merge_empty_partials(cuda):
     assert torch.equal(out.cpu(), o2.float()) and torch.equal(lse.cpu(), l2)
 
 
-def test_ring_sweep_equals_full_attention(cuda):
+@pytest.mark.parametrize("fused", [True, False])
+def test_ring_sweep_equals_full_attention(cuda, fused):
     # BASELINE config 3 in miniature, ragged like 14882 = 116*128 + 34: 8 blocks of 290 keys
     B, H, Sq, D, nblk, blk = 1, 4, 290, 128, 8, 290
     q, k, v = inputs.qkv(B, H, Sq, nblk * blk, D, seed=3)
     ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
     kb = [k[:, :, i * blk : (i + 1) * blk].contiguous().to(cuda) for i in range(nblk)]
     vb = [v[:, :, i * blk : (i + 1) * blk].contiguous().to(cuda) for i in range(nblk)]
-    out, lse = paraattention_amd.ring_sweep(q.to(cuda), kb, vb)
+    out, lse = paraattention_amd.ring_sweep(q.to(cuda), kb, vb, fused=fused)
     assert out.dtype == torch.bfloat16
     np.testing.assert_allclose(lse.cpu().numpy(), ref_lse, atol=1e-3)
     np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+
+
+def test_fused_accumulate_steps(cuda, monkeypatch):
+    """attention_forward_accumulate_ / _final against the oracle's merge of the oracle's partials, on a grid that
+    takes the key-split tail (so the split merge folds the accumulator too), with a strided query."""
+    from oracle import merge as omerge
+    from paraattention_amd import _lib
+
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    B, H, D = 1, 8, 128
+    Sq = (cus // (B * H) + 3) * 256 - 77
+    blks = [64 * 40 + 5, 64 * 33, 64 * 47 + 63]
+    q, k, v = inputs.qkv(B, H, Sq, sum(blks), D, seed=5)
+    qd = q.to(cuda).transpose(1, 2).contiguous().transpose(1, 2)
+    ks, vs = k.split(blks, 2), v.split(blks, 2)
+    assert _lib.load().pa_attn_fwd_workspace_bytes(B, H, Sq, blks[0], D, _lib.strides3(ks[0]), _lib.strides3(vs[0])) > 0
+    acc = torch.full((B, H, Sq, D), float("nan"), device=cuda)       # first=True must not read it
+    acc_l = torch.full((B, H, Sq), float("nan"), device=cuda)
+    rows = torch.cat([torch.arange(0, 40), torch.arange(Sq - 300, Sq)])  # unsplit head and split tail tiles
+    parts = [oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), kk.float().numpy(), vv.float().numpy()) for kk, vv in zip(ks, vs)]
+    for i in range(2):
+        torch.ops.para_attn.attention_forward_accumulate_(acc, acc_l, qd, ks[i].to(cuda), vs[i].to(cuda), i == 0)
+        ro, rl = omerge.merge_all([p[0] for p in parts[: i + 1]], [p[1] for p in parts[: i + 1]])
+        np.testing.assert_allclose(acc_l[:, :, rows].cpu().numpy(), rl, atol=1e-3)
+        np.testing.assert_allclose(acc[:, :, rows].cpu().numpy(), ro, atol=2e-2, rtol=2e-2)
+    before = acc.clone()
+    out = torch.ops.para_attn.attention_forward_accumulate_final(acc, acc_l, qd, ks[2].to(cuda), vs[2].to(cuda))
+    assert out.dtype == torch.bfloat16 and torch.equal(acc, before)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), k.float().numpy(), v.float().numpy())
+    np.testing.assert_allclose(acc_l[:, :, rows].cpu().numpy(), ref_lse, atol=1e-3)
+    np.testing.assert_allclose(out[:, :, rows].float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+    # unsplit launch gives the same (to rounding)
+    monkeypatch.setenv("PARAATTN_NO_SPLIT", "1")
+    acc_l2 = acc_l.clone()
+    torch.ops.para_attn.attention_forward_accumulate_(acc, acc_l2, qd, ks[0].to(cuda), vs[0].to(cuda), True)
+    torch.ops.para_attn.attention_forward_accumulate_(acc, acc_l2, qd, ks[1].to(cuda), vs[1].to(cuda))
+    out2 = torch.ops.para_attn.attention_forward_accumulate_final(acc, acc_l2, qd, ks[2].to(cuda), vs[2].to(cuda))
+    assert (out2.float() - out.float()).abs().max().item() <= 2e-2 and (acc_l2 - acc_l).abs().max().item() <= 1e-4
+    # unsupported shapes say so
+    q64, k64, v64 = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 64))
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward_accumulate_(torch.zeros(1, 1, 16, 64, device=cuda), torch.zeros(1, 1, 16, device=cuda), q64, k64, v64, True)
 
 
 def test_ring_sweep_full_shape_sampled(cuda):
