@@ -7,7 +7,7 @@ resident in HBM (a call = the attention kernel plus the 8 us merge of its key-sp
 against) on a bounded sample of the same workload; ``extras`` holds the bandwidth-bound kernels
 (ring merge step, FBCache reduction) against the HBM peak and the block-sparse mode.
 
-``--only {attn,merge,fbcache,sparse}`` runs a single kernel's loop (what the rocprofv3 summaries
+``--only {attn,merge,fbcache,taylorseer,sparse}`` runs a single kernel's loop (what the rocprofv3 summaries
 under profiles/ were taken with).
 """
 import argparse
@@ -100,6 +100,20 @@ def bench_fbcache(dev, steps=20, warmup=3):
     return r
 
 
+def bench_taylorseer(dev, steps=20, warmup=3):
+    import torch
+
+    # cache-hit step with TaylorSeer on: value of 3 stored orders + hidden states, one pass
+    shape = (1, 32760, 5120)
+    g = torch.Generator().manual_seed(5)
+    ds = [torch.randn(shape, generator=g, dtype=torch.bfloat16).to(dev) for _ in range(3)]
+    hidden = torch.randn(shape, generator=g, dtype=torch.bfloat16).to(dev)
+    op = torch.ops.para_attn.taylorseer_value
+    ms, _ = _time_calls(lambda: op(ds, 2, hidden), steps, warmup)
+    return _hbm("taylorseer", "TaylorSeer cache hit: 3 stored orders + hidden states, bf16 [1,32760,5120], one pass",
+                5 * 2 * hidden.numel(), ms)
+
+
 def bench_sparse(dev, steps=5, warmup=2):
     import torch
 
@@ -178,7 +192,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only", choices=["attn", "merge", "fbcache", "sparse", "copy"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "fbcache", "taylorseer", "sparse", "copy"], default=None,
                     help="profiling aid: run just one kernel's timed loop and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -193,8 +207,9 @@ def main():
     _lib.load()  # no fallback: a missing library is an error
     dev = torch.device("cuda:0")
 
-    if args.only in ("merge", "fbcache", "sparse", "copy"):
-        fn = {"merge": bench_merge, "fbcache": bench_fbcache, "sparse": bench_sparse, "copy": bench_copy}[args.only]
+    if args.only in ("merge", "fbcache", "taylorseer", "sparse", "copy"):
+        fn = {"merge": bench_merge, "fbcache": bench_fbcache, "taylorseer": bench_taylorseer, "sparse": bench_sparse,
+              "copy": bench_copy}[args.only]
         print(json.dumps({args.only: fn(dev, args.steps, args.warmup)}))
         return
 
@@ -237,6 +252,7 @@ def main():
         result["extras"] = {
             "merge_lse": bench_merge(dev),
             "fbcache_residual_diff": bench_fbcache(dev),
+            "taylorseer_value": bench_taylorseer(dev),
             "block_sparse": bench_sparse(dev),
         }
     if not args.no_cpu_baseline:

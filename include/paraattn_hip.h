@@ -227,6 +227,31 @@ PA_API int pa_fbcache_residual_ratio(const void* hidden, const void* hidden0, co
 PA_API int pa_fbcache_apply_residual(const void* resid, const void* hidden, void* out, int dtype,
                               int64_t n, void* stream);
 
+/*
+ * TaylorSeer finite differences (src/para_attn/first_block_cache/taylorseer.py:29-38,
+ * approximate_derivative): with x_0 = y, for i < n
+ *     cur[i] = (x_i - prev[i]) / window,   x_{i+1} = cur[i]
+ * in one pass, with torch's eager rounding for 16-bit tensors (the difference
+ * and the quotient are each rounded to `dtype`; true division).  prev and cur
+ * are host arrays of n device pointers (n <= 4) to contiguous tensors of numel
+ * elements, 16-byte aligned; cur[i] must not alias y or prev[j].
+ */
+PA_API int pa_taylorseer_update(const void* y, const void* const* prev, void* const* cur, int n,
+                         int dtype, int64_t numel, float window, void* stream);
+
+/*
+ * TaylorSeer extrapolation (taylorseer.py:40-48, approximate_value):
+ *     out = 0;  out += coef[i] * deriv[i] * pw[i]   for i < m
+ * with coef[i] = (float)(1 / i!) and pw[i] = (float)(elapsed ** i) supplied by
+ * the caller (host arrays of m floats, m <= 5), every product and sum rounded
+ * to `dtype` as torch's eager ops round them.  hidden != NULL additionally
+ * gives out = hidden + value: the cache-hit path of
+ * src/para_attn/first_block_cache/utils.py:239-243 in the same pass.  deriv is
+ * a host array of m device pointers.  out may alias hidden.
+ */
+PA_API int pa_taylorseer_value(const void* const* deriv, int m, const float* coef, const float* pw,
+                        const void* hidden, void* out, int dtype, int64_t numel, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

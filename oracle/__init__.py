@@ -13,6 +13,7 @@ torch==2.6.0 in its README.md:153 and torch==2.5.0 in quick_install.sh:3):
                 _context_parallel/_attention.py:138-223)
   sparse.py     src/para_attn/sparse_attn.py:74-278 (ranges, run scan, merges)
   fbcache.py    src/para_attn/first_block_cache/utils.py:220-234, 269-286
+  taylorseer.py src/para_attn/first_block_cache/taylorseer.py:4-64 (finite differences, extrapolation)
   inputs.py     seeded generators of the benchmark configurations
 
 Pinning status (what fixes each function besides its own formula):
@@ -26,6 +27,10 @@ Pinning status (what fixes each function besides its own formula):
   sparse.struct_sparse_f64     the -inf-masked dense closed form
   fbcache.residual_diff_ratio  torch's bf16/fp16 CPU op chain on fixtures incl.
                                near-threshold cases; decision-table known answers
+  taylorseer.finite_differences torch's bf16/fp16/fp32 CPU op chain evaluating the
+  / extrapolate / TaylorSeer   reference's expressions, bit for bit; closed forms (a linear
+                               sequence is extrapolated exactly, t^2 with unit window gives
+                               (t+e)^2 - e); the compute/skip schedule by enumeration
 The reference's own tests hold no golden vectors for this path
 (tests/ops/test_ops.py:62 compares the output with itself), so none are used.
 """

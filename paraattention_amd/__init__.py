@@ -6,11 +6,12 @@ fallback.
 """
 from . import config  # noqa: F401
 from . import ops  # noqa: F401  (registers torch.ops.para_attn.*)
-from . import fbcache, merge, sparse  # noqa: F401
+from . import fbcache, merge, sparse, taylorseer  # noqa: F401
 from .merge import SDPAMerger, ring_sweep  # noqa: F401
+from .taylorseer import TaylorSeer  # noqa: F401
 from .sparse import StructSparseAttnMode, struct_sparse_attn_func  # noqa: F401
 
 __all__ = [
-    "config", "ops", "merge", "sparse", "fbcache",
+    "config", "ops", "merge", "sparse", "fbcache", "taylorseer", "TaylorSeer",
     "SDPAMerger", "ring_sweep", "StructSparseAttnMode", "struct_sparse_attn_func",
 ]

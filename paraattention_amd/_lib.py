@@ -30,6 +30,8 @@ _i64 = ctypes.c_int64
 _f = ctypes.c_float
 _sz = ctypes.c_size_t
 _strides = ctypes.POINTER(ctypes.c_int64)
+_ptrs = ctypes.POINTER(ctypes.c_void_p)  # host array of device pointers
+_floats = ctypes.POINTER(ctypes.c_float)  # host array
 
 # name -> (restype, argtypes); mirrors include/paraattn_hip.h declaration by declaration
 SIGNATURES = {
@@ -58,6 +60,8 @@ SIGNATURES = {
     "pa_blocksparse_workspace_bytes": (_sz, [_i, _i, _i]),
     "pa_blocksparse_build_runs": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "pa_merge_lse": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _i64, _i, _vp]),
+    "pa_taylorseer_update": (_i, [_vp, _ptrs, _ptrs, _i, _i, _i64, _f, _vp]),
+    "pa_taylorseer_value": (_i, [_ptrs, _i, _floats, _floats, _vp, _vp, _i, _i64, _vp]),
     "pa_fbcache_absdiff_ratio": (
         _i,
         [_vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp],

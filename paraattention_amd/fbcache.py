@@ -1,9 +1,9 @@
 """First Block Cache decision path with the reference's function names
 (src/para_attn/first_block_cache/utils.py:12-120, 193-295): the cache context,
 the gates of ``get_can_use_cache`` and ``are_two_tensors_similar``, whose
-seven-launch reduction is one kernel here.  Only what the decision needs is
-kept; TaylorSeer, the diffusers adapters and the block orchestration are not
-part of this package.
+seven-launch reduction is one kernel here, and the TaylorSeer variant of the
+cached residual (utils.py:297-312).  The diffusers adapters and the block
+orchestration are not part of this package.
 """
 import contextlib
 import dataclasses
@@ -12,6 +12,7 @@ from typing import Any, Dict, Optional, Union
 import torch
 
 from . import ops
+from .taylorseer import TaylorSeer
 
 
 @dataclasses.dataclass
@@ -24,9 +25,24 @@ class CacheContext:
     enable_alter_cache: bool = False
     num_inference_steps: int = -1
     warmup_steps: int = 0
+    enable_taylorseer: bool = False
+    taylorseer_kwargs: Dict[str, Any] = dataclasses.field(default_factory=dict)
+    taylorseer: Optional[TaylorSeer] = None
+    alter_taylorseer: Optional[TaylorSeer] = None
     buffers: Dict[str, Any] = dataclasses.field(default_factory=dict)
     executed_steps: int = 0
     is_alter_cache: bool = True
+
+    def __post_init__(self):
+        if self.enable_taylorseer:
+            self.taylorseer = TaylorSeer(**self.taylorseer_kwargs)
+            if self.enable_alter_cache:
+                self.alter_taylorseer = TaylorSeer(**self.taylorseer_kwargs)
+
+    def get_taylorseer(self):
+        if self.enable_alter_cache and self.is_alter_cache:
+            return self.alter_taylorseer
+        return self.taylorseer
 
     def get_residual_diff_threshold(self):
         if self.enable_alter_cache and self.is_alter_cache and self.alter_residual_diff_threshold is not None:
@@ -59,6 +75,8 @@ class CacheContext:
             self.is_alter_cache = not self.is_alter_cache
             if not self.is_alter_cache:
                 self.executed_steps += 1
+        if self.enable_taylorseer:
+            self.get_taylorseer().mark_step_begin()
 
     def get_current_step(self):
         return self.executed_steps - 1
@@ -179,6 +197,10 @@ def first_block_step(hidden_states, original_hidden_states, parallelized=False):
 def apply_prev_hidden_states_residual(hidden_states, encoder_hidden_states=None):
     """Cache hit (utils.py:237-259): add the stored residuals back."""
     ctx = _ctx()
+    if ctx.enable_taylorseer:
+        # utils.py:239-243: the extrapolated residual plus the hidden states, one pass; the
+        # encoder residual is not kept in this mode (utils.py:314-317) and stays untouched
+        return ctx.get_taylorseer().approximate_value_plus(hidden_states), encoder_hidden_states
     res = ctx.get_buffer("hidden_states_residual")
     assert res is not None, "hidden_states_residual must be set before"
     hidden_states = ops.fbcache_apply_residual(res, hidden_states)
@@ -187,3 +209,46 @@ def apply_prev_hidden_states_residual(hidden_states, encoder_hidden_states=None)
         assert eres is not None, "encoder_hidden_states_residual must be set before"
         encoder_hidden_states = ops.fbcache_apply_residual(eres, encoder_hidden_states)
     return hidden_states, encoder_hidden_states
+
+
+@torch.compiler.disable
+def is_taylorseer_enabled():
+    return _ctx().enable_taylorseer
+
+
+@torch.compiler.disable
+def get_taylorseer():
+    return _ctx().get_taylorseer()
+
+
+@torch.compiler.disable
+def set_hidden_states_residual(hidden_states_residual):
+    """utils.py:297-303."""
+    ctx = _ctx()
+    if ctx.enable_taylorseer:
+        ctx.get_taylorseer().update(hidden_states_residual)
+    else:
+        ctx.set_buffer("hidden_states_residual", hidden_states_residual)
+
+
+@torch.compiler.disable
+def get_hidden_states_residual():
+    """utils.py:306-312."""
+    ctx = _ctx()
+    if ctx.enable_taylorseer:
+        return ctx.get_taylorseer().approximate_value()
+    return ctx.get_buffer("hidden_states_residual")
+
+
+@torch.compiler.disable
+def set_encoder_hidden_states_residual(encoder_hidden_states_residual):
+    """utils.py:314-318."""
+    ctx = _ctx()
+    if ctx.enable_taylorseer:
+        return
+    ctx.set_buffer("encoder_hidden_states_residual", encoder_hidden_states_residual)
+
+
+@torch.compiler.disable
+def get_encoder_hidden_states_residual():
+    return _ctx().get_buffer("encoder_hidden_states_residual")

@@ -19,10 +19,11 @@ torch elementwise calls:
   attention_forward_block_sparse               (sparse_attn.py:74-278)
   fbcache_residual_diff                        (first_block_cache/utils.py:228-233)
   fbcache_first_residual_diff, fbcache_apply_residual (utils.py:359, 237-259)
+  taylorseer_derivatives, taylorseer_value     (first_block_cache/taylorseer.py:29-48)
 """
 import ctypes
 import math
-from typing import Optional, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -605,3 +606,77 @@ def fbcache_apply_residual(residual: torch.Tensor, hidden: torch.Tensor) -> torc
 @torch.library.register_fake("para_attn::fbcache_apply_residual")
 def _(residual, hidden):
     return hidden.new_empty(hidden.shape)
+
+
+# ---------------------------------------------------------------------------------
+# TaylorSeer
+# ---------------------------------------------------------------------------------
+def _flat_same(tensors, what):
+    t0 = tensors[0]
+    if t0.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"{what}: dtype {t0.dtype} not supported")
+    out = []
+    for t in tensors:
+        if t.shape != t0.shape or t.dtype != t0.dtype or t.device != t0.device:
+            raise ValueError(f"{what}: tensors must share shape, dtype and device")
+        out.append(t if t.is_contiguous() and t.data_ptr() % 16 == 0 else t.contiguous().clone())
+    return out
+
+
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+@torch.library.custom_op("para_attn::taylorseer_derivatives", mutates_args=(), device_types=("cuda",))
+def taylorseer_derivatives(y: torch.Tensor, prev: List[torch.Tensor], window: float) -> List[torch.Tensor]:
+    """The finite differences of TaylorSeer.approximate_derivative
+    (src/para_attn/first_block_cache/taylorseer.py:29-38) in one pass: with x0 = y,
+    returns [x1, ..., xn] where x_{i+1} = (x_i - prev[i]) / window, rounded as torch's
+    eager ops round (difference, then quotient)."""
+    n = len(prev)
+    if n == 0:
+        return []
+    ts = _flat_same([y] + list(prev), "taylorseer_derivatives")
+    cur = [torch.empty(y.shape, dtype=y.dtype, device=y.device) for _ in range(n)]
+    lib = _lib.load()
+    with torch.cuda.device(y.device):
+        rc = lib.pa_taylorseer_update(
+            _ptr(ts[0]), _ptr_array(ts[1:]), _ptr_array(cur), n, _DTYPE_CODE[y.dtype], y.numel(), float(window),
+            _stream_ptr(y.device),
+        )
+    _lib.check(rc, "pa_taylorseer_update")
+    return cur
+
+
+@torch.library.register_fake("para_attn::taylorseer_derivatives")
+def _(y, prev, window):
+    return [torch.empty_like(y) for _ in prev]
+
+
+@torch.library.custom_op("para_attn::taylorseer_value", mutates_args=(), device_types=("cuda",))
+def taylorseer_value(derivs: List[torch.Tensor], elapsed: int, hidden: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """TaylorSeer.approximate_value (taylorseer.py:40-48): sum over the stored orders of
+    (1 / i!) * derivs[i] * elapsed**i, each product and partial sum rounded as torch's eager
+    ops round; with ``hidden``, the cache-hit add ``value + hidden`` of
+    src/para_attn/first_block_cache/utils.py:239-243 in the same pass."""
+    m = len(derivs)
+    if m == 0:
+        raise ValueError("taylorseer_value: no stored derivative")
+    ts = _flat_same(list(derivs) + ([hidden] if hidden is not None else []), "taylorseer_value")
+    d0 = ts[0]
+    out = torch.empty(d0.shape, dtype=d0.dtype, device=d0.device)
+    coef = (ctypes.c_float * m)(*[1 / math.factorial(i) for i in range(m)])
+    pw = (ctypes.c_float * m)(*[float(elapsed**i) for i in range(m)])
+    lib = _lib.load()
+    with torch.cuda.device(d0.device):
+        rc = lib.pa_taylorseer_value(
+            _ptr_array(ts[:m]), m, coef, pw, _ptr(ts[m]) if hidden is not None else None, _ptr(out),
+            _DTYPE_CODE[d0.dtype], d0.numel(), _stream_ptr(d0.device),
+        )
+    _lib.check(rc, "pa_taylorseer_value")
+    return out
+
+
+@torch.library.register_fake("para_attn::taylorseer_value")
+def _(derivs, elapsed, hidden=None):
+    return torch.empty_like(derivs[0])

@@ -3,6 +3,8 @@
 Expected values come from torch's CPU library routines (the arithmetic the reference delegates to):
   fbcache_*   eager bf16/fp16 ops of are_two_tensors_similar (src/para_attn/first_block_cache/utils.py:228-233)
   attention_* torch CPU SDPA (bf16 out + fp32 LSE), the oracle of src/para_attn/ops/__init__.py:160-179
+  taylorseer_* eager ops evaluating the expressions of src/para_attn/first_block_cache/taylorseer.py:35,45
+              and the cache-hit add of first_block_cache/utils.py:242
   merge_*     torch _SDPAMerger (torch/distributed/tensor/experimental/_context_parallel/_attention.py:138-223)
 The reference holds no golden vectors of its own for these ops (tests/ops/test_ops.py:62 is a tautology).
 """
@@ -81,8 +83,45 @@ def merge():
     np.savez_compressed(os.path.join(HERE, "merge_cases.npz"), **arrays)
 
 
+def taylorseer():
+    import math
+
+    arrays, cases = {}, []
+    g = torch.Generator().manual_seed(23)
+    specs = [  # name, dtype, shape, orders of difference / stored orders, window, elapsed
+        ("bf16_w1", torch.bfloat16, (1, 37, 23), 2, 1, 1),
+        ("bf16_w3", torch.bfloat16, (1, 37, 23), 2, 3, 2),
+        ("bf16_o4", torch.bfloat16, (2, 16, 40), 4, 5, 3),
+        ("f16_w3", torch.float16, (1, 37, 23), 2, 3, 2),
+        ("f32_w3", torch.float32, (1, 9, 7), 3, 3, 4),
+    ]
+    for name, dtype, shape, n, window, elapsed in specs:
+        y = (torch.randn(shape, generator=g) * 2).to(dtype)
+        prev = [(torch.randn(shape, generator=g) * (2.0 / (i + 1))).to(dtype) for i in range(n)]
+        hidden = torch.randn(shape, generator=g).to(dtype)
+        # approximate_derivative (taylorseer.py:33-35)
+        cur = [y]
+        for i in range(n):
+            cur.append((cur[i] - prev[i]) / window)
+        # approximate_value (taylorseer.py:42-47) over the orders just built
+        output = 0
+        for i, derivative in enumerate(cur):
+            output += (1 / math.factorial(i)) * derivative * (elapsed**i)
+        applied = output + hidden  # utils.py:242
+        enc = bf16_bits if dtype == torch.bfloat16 else (lambda t: t.numpy())
+        arrays[name + "_y"], arrays[name + "_hidden"] = enc(y), enc(hidden)
+        for i in range(n):
+            arrays[f"{name}_prev{i}"], arrays[f"{name}_cur{i + 1}"] = enc(prev[i]), enc(cur[i + 1])
+        arrays[name + "_value"], arrays[name + "_applied"] = enc(output), enc(applied)
+        cases.append({"name": name, "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
+                      "n": n, "window": window, "elapsed": elapsed})
+    arrays["cases"] = np.array(json.dumps(cases))
+    np.savez_compressed(os.path.join(HERE, "taylorseer_cases.npz"), **arrays)
+
+
 if __name__ == "__main__":
     fbcache()
+    taylorseer()
     attention()
     merge()
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith((".npz", ".json"))))

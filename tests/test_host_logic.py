@@ -136,3 +136,36 @@ def test_merger_refuses_partial_mode():
     m = paraattention_amd.SDPAMerger(True, 2)
     with pytest.raises(NotImplementedError):
         m.step(torch.zeros(1, 1, 4, 8), torch.zeros(1, 1, 4), partial=True)
+
+
+def test_cache_context_builds_taylorseers():
+    """utils.py:39-43, 90-97: one TaylorSeer, or two with the alternating cache; mark_step_begin advances the active one."""
+    from paraattention_amd import fbcache
+    from paraattention_amd.taylorseer import TaylorSeer
+
+    ctx = fbcache.create_cache_context(enable_taylorseer=True, taylorseer_kwargs={"n_derivatives": 1, "warmup_steps": 2})
+    assert isinstance(ctx.taylorseer, TaylorSeer) and ctx.alter_taylorseer is None and ctx.taylorseer.ORDER == 2
+    ctx.mark_step_begin()
+    ctx.mark_step_begin()
+    assert ctx.taylorseer.current_step == 1 and ctx.get_taylorseer() is ctx.taylorseer
+    ctx = fbcache.create_cache_context(enable_taylorseer=True, enable_alter_cache=True)
+    assert ctx.alter_taylorseer is not None
+    ctx.mark_step_begin()  # -> not alter: the plain one advances
+    assert ctx.get_taylorseer() is ctx.taylorseer and ctx.taylorseer.current_step == 0 and ctx.alter_taylorseer.current_step == -1
+    ctx.mark_step_begin()  # -> alter
+    assert ctx.get_taylorseer() is ctx.alter_taylorseer and ctx.alter_taylorseer.current_step == 0
+    assert fbcache.create_cache_context().taylorseer is None
+
+
+def test_taylorseer_schedule_and_limits():
+    """taylorseer.py:21-27 (schedule) with the reference's own self-test settings; the kernels take at most 4 orders."""
+    import pytest
+
+    from paraattention_amd.taylorseer import TaylorSeer
+
+    ts = TaylorSeer(n_derivatives=2, warmup_steps=2, skip_interval_steps=2)
+    assert [ts.should_compute_full(s) for s in range(8)] == [True, True, False, True, False, True, False, True]
+    assert TaylorSeer(compute_step_map=[False, True]).should_compute_full(1) is True
+    assert ts.approximate_value() == 0  # nothing stored: the reference's empty sum
+    with pytest.raises(NotImplementedError):
+        TaylorSeer(n_derivatives=5)
