@@ -114,7 +114,7 @@ def bench_taylorseer(dev, steps=20, warmup=3):
                 5 * 2 * hidden.numel(), ms)
 
 
-def bench_sparse(dev, steps=5, warmup=2):
+def bench_sparse(dev, steps=10, warmup=5):
     import torch
 
     from oracle import inputs

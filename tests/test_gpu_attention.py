@@ -231,6 +231,28 @@ def test_key_split_tail(cuda, bm, monkeypatch):
     monkeypatch.delenv("PARAATTN_BM")
 
 
+def test_key_rows_spread_over_4gib(cuda):
+    """K and V whose rows lie 1 MiB apart span more than 4 GiB per head: beyond the 32-bit offsets of the
+    pipelined kernel, so the launch must pick the kernel without that limit (a wrong pick reads zeros)."""
+    B, H, Sq, Skv, D = 1, 1, 200, 4100, 128
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=31)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    stride = 1 << 19  # elements between consecutive key rows
+    big = torch.empty(2, Skv * stride, dtype=torch.bfloat16, device=cuda)
+    kd = big[0].as_strided((B, H, Skv, D), (0, 0, stride, 1))
+    vd = big[1].as_strided((B, H, Skv, D), (0, 0, stride, 1))
+    kd.copy_(k.to(cuda))
+    vd.copy_(v.to(cuda))
+    assert (Skv - 1) * stride * 2 >= 1 << 32
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), kd, vd)
+    _check(out, lse, ref_out, ref_lse, "rows 1 MiB apart")
+    with pytest.raises(NotImplementedError):  # the fused ring step has no such fallback and says so
+        torch.ops.para_attn.attention_forward_accumulate_(
+            torch.empty(B, H, Sq, D, device=cuda), torch.empty(B, H, Sq, device=cuda), q.to(cuda), kd, vd, True)
+    del big, kd, vd
+    torch.cuda.empty_cache()
+
+
 def test_unsupported_raise(cuda):
     q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 128))
     with pytest.raises(NotImplementedError):
