@@ -1037,17 +1037,32 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage A ---------------------------------------------------------------------------------
-    // The 32 scores of S(j) per lane are exponentiated 24 in stage A and 8 in the first half of
-    // stage B (P of keys 32..63 is only needed by the last 8 MFMAs), which keeps the VALU work
+    // The 32 scores of S(j) per lane are exponentiated over the 16 groups of stage A and the first
+    // 6 of stage B (P of keys 32..63 is only needed by the last 8 MFMAs), which keeps the VALU work
     // per MFMA below the MFMA's own 32 cycles.  The row sum adds the fp32 values before rounding
     // (summing the rounded ones costs up to 3e-3 of LSE on peaked rows).
     uint32_t pk0[8], pk1[8];
     float lsum = 0.f;
-    auto expo = [&](const floatx16& cs, uint32_t* pk, int i) {  // scores 2i, 2i+1 -> packed pair i
-      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cs[2 * i], c, -m_run));
-      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cs[2 * i + 1], c, -m_run));
-      lsum += p0 + p1;
-      pk[i] = T::pack2(p0, p1);
+    // Pair n of the 16 score pairs (0..7: keys 0..31, 8..15: keys 32..63) goes through three
+    // steps in three consecutive slots, so that no instruction of a slot waits for another of
+    // the same slot: scale and shift, exponential, sum and pack.
+    float tf[2][2], te[2][2];
+    auto expo_slot = [&](int n) {
+      if (n >= 2 && n < 18) {
+        const int j = n - 2;
+        lsum += te[j & 1][0] + te[j & 1][1];
+        (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
+      }
+      if (n >= 1 && n < 17) {
+        const int j = n - 1;
+        te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
+        te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
+      }
+      if (n < 16) {
+        const floatx16& cs = n < 8 ? c0 : c1;
+        tf[n & 1][0] = __builtin_fmaf(cs[2 * (n & 7)], c, -m_run);
+        tf[n & 1][1] = __builtin_fmaf(cs[2 * (n & 7) + 1], c, -m_run);
+      }
     };
 #pragma unroll
     for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
@@ -1057,14 +1072,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       if (g < IPW) dma_k1(par, n_nx2, g);                      // K(j+2) takes the buffer K(j) has left
       else if (g < 2 * IPW) dma_v1(par ^ 1, n_nxt, g - IPW);  // V(j+1) takes the buffer V(j-1) has left
       f[g] = read_k(tKn, 1, g);
-      expo(c0, pk0, g);
+      expo_slot(g);
       __builtin_amdgcn_sched_barrier(0);  // keep the groups in this order
     }
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
       sn1 = T::mfma32(f[g], qf[g], sn1);
       f[g] = read_vt(tV, 0, g >> 2, g & 3);  // V(j), keys 0..31, takes the slot over
-      if (g < 4) expo(c1, pk1, g);
+      if (g < 4) expo_slot(8 + g);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (v_nxt < BN) mask_tail(sn0, sn1, v_nxt);  // ragged (or absent) tile j+1
@@ -1081,8 +1096,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
         f[g] = read_vt(tV, 1, cc, db);  // keys 32..63
-        if (g < 4) expo(c1, pk1, 4 + g);
-        else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
+        if (g < 6) expo_slot(12 + g);
+        if (g < 4) {
+        } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
         else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
         __builtin_amdgcn_sched_barrier(0);
       }
