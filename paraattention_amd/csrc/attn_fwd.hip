@@ -1103,7 +1103,6 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    l_run += lsum;
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
@@ -1116,6 +1115,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    l_run += lsum;
     mx = across(fmaxf(mxa, mxb));
 
     // slide the tile window
