@@ -114,6 +114,27 @@ def bench_taylorseer(dev, steps=20, warmup=3):
                 5 * 2 * hidden.numel(), ms)
 
 
+def bench_ring(dev, steps=5, warmup=2):
+    import torch
+
+    import paraattention_amd
+
+    # one rank's ring pass: Q block of 14882 tokens x 24 heads against 8 KV blocks, merge folded into the kernel
+    B, H, S, D, nblk = 1, 24, 14882, 128, 8
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(B, H, S, D, generator=g).bfloat16().to(dev)
+    kb = [torch.randn(B, H, S, D, generator=g).bfloat16().to(dev) for _ in range(nblk)]
+    vb = [torch.randn(B, H, S, D, generator=g).bfloat16().to(dev) for _ in range(nblk)]
+    ms, _ = _time_calls(lambda: paraattention_amd.ring_sweep(q, kb, vb), steps, warmup)
+    flops = 4.0 * B * H * S * S * nblk * D
+    tf = flops / (ms * 1e-3) / 1e12
+    return {
+        "workload": "ring sweep: Q block [1,24,14882,128] bf16 against 8 KV blocks of 14882 keys, fused accumulate",
+        "bound": "mfma", "flop_per_sweep": flops, "ms_per_sweep": round(ms, 4), "launches_per_sweep": nblk,
+        "achieved": round(tf, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4),
+    }
+
+
 def bench_sparse(dev, steps=10, warmup=5):
     import torch
 
@@ -254,6 +275,7 @@ def main():
             "fbcache_residual_diff": bench_fbcache(dev),
             "taylorseer_value": bench_taylorseer(dev),
             "block_sparse": bench_sparse(dev),
+            "ring_sweep": bench_ring(dev),
         }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(q, k, v)
