@@ -1021,7 +1021,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
 
     // first fragments of K(j+1) on their way while the maximum is settled
 #pragma unroll
-    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, 0, dc);
+    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
 
     const float mx_s = mx * c;
     if (__any(mx_s > m_run + RESCALE_SLACK)) {
@@ -1068,16 +1068,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
-      sn0 = T::mfma32(f[g], qf[g], sn0);
+      // the two halves of S(j+1) alternate, so that no MFMA waits for the one just issued
+      if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
+      else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
       if (g < IPW) dma_k1(par, n_nx2, g);                      // K(j+2) takes the buffer K(j) has left
       else if (g < 2 * IPW) dma_v1(par ^ 1, n_nxt, g - IPW);  // V(j+1) takes the buffer V(j-1) has left
-      f[g] = read_k(tKn, 1, g);
+      f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
       expo_slot(g);
       __builtin_amdgcn_sched_barrier(0);  // keep the groups in this order
     }
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
-      sn1 = T::mfma32(f[g], qf[g], sn1);
+      if (g & 1) sn1 = T::mfma32(f[g], qf[4 + (g >> 1)], sn1);
+      else sn0 = T::mfma32(f[g], qf[4 + (g >> 1)], sn0);
       f[g] = read_vt(tV, 0, g >> 2, g & 3);  // V(j), keys 0..31, takes the slot over
       if (g < 4) expo_slot(8 + g);
       __builtin_amdgcn_sched_barrier(0);
