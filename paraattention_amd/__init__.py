@@ -6,12 +6,14 @@ fallback.
 """
 from . import config  # noqa: F401
 from . import ops  # noqa: F401  (registers torch.ops.para_attn.*)
-from . import fbcache, merge, sparse, taylorseer  # noqa: F401
+from . import fbcache, interface, merge, sparse, taylorseer  # noqa: F401
+from .interface import SparseKVAttnMode, UnifiedAttnMode, sparse_kv_attn_func  # noqa: F401
 from .merge import SDPAMerger, ring_sweep  # noqa: F401
 from .taylorseer import TaylorSeer  # noqa: F401
 from .sparse import StructSparseAttnMode, struct_sparse_attn_func  # noqa: F401
 
 __all__ = [
-    "config", "ops", "merge", "sparse", "fbcache", "taylorseer", "TaylorSeer",
+    "config", "ops", "merge", "sparse", "fbcache", "taylorseer", "TaylorSeer", "interface",
+    "UnifiedAttnMode", "SparseKVAttnMode", "sparse_kv_attn_func",
     "SDPAMerger", "ring_sweep", "StructSparseAttnMode", "struct_sparse_attn_func",
 ]

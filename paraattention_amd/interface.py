@@ -1,0 +1,159 @@
+"""The reference's interception mode for plain attention calls, for one GPU
+(src/para_attn/para_attn_interface.py:395-479).
+
+``with UnifiedAttnMode(): F.scaled_dot_product_attention(q, k, v)`` walks the reference's three
+stages (ulysses, ring, none).  On one GPU the first two pass through
+(para_attn_interface.py:62-63, 217-226), and the last one ends in ``attn_func`` if given, in
+``para_attn::attention_forward`` when ``config.attention.force_dispatch_to_custom_ops`` is set
+(:468-470) or -- where the reference would call aten's SDPA, which has no kernel of its own on
+this GPU -- when the call is one the HIP kernel takes; any other call goes to
+``F.scaled_dot_product_attention`` untouched.  A mesh of more than one rank is refused.
+"""
+import contextlib
+
+import torch
+import torch.nn.functional as F
+from torch.overrides import TorchFunctionMode
+
+from . import config, ops
+
+_SDPA_ARGS = ("query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale", "enable_gqa")
+
+
+def _bind(args, kwargs):
+    bound = dict(zip(_SDPA_ARGS, args))
+    bound.update(kwargs)
+    return bound
+
+
+def kernel_takes(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None, enable_gqa=False):
+    """Whether ``para_attn::attention_forward`` computes this SDPA call on the GPU."""
+    if not (isinstance(query, torch.Tensor) and query.is_cuda and query.ndim == 4 and key.ndim == 4 and value.ndim == 4):
+        return False
+    if query.dtype not in (torch.bfloat16, torch.float16) or key.dtype != query.dtype or value.dtype != query.dtype:
+        return False
+    if dropout_p != 0.0 or is_causal or enable_gqa or query.shape[1] != key.shape[1]:
+        return False
+    if query.shape[-1] not in (64, 128) or value.shape[-1] != query.shape[-1]:
+        return False
+    if query.requires_grad or key.requires_grad or value.requires_grad:
+        return False  # forward only, like the reference's ops (src/para_attn/ops/__init__.py:203-211)
+    if attn_mask is not None:
+        # a boolean mask over keys only, the same for every query row
+        if attn_mask.dtype != torch.bool or attn_mask.ndim != 4 or attn_mask.shape[-2] != 1 or attn_mask.shape[1] != 1:
+            return False
+    return True
+
+
+def _world_size(mesh):
+    if mesh is None:
+        return 1
+    if hasattr(mesh, "size"):
+        return mesh.size() if callable(mesh.size) else mesh.size
+    raise TypeError("mesh must be a ProcessGroup or DeviceMesh")
+
+
+class UnifiedAttnMode(TorchFunctionMode):
+    disabled = False
+
+    @torch.compiler.disable
+    def __init__(self, mesh=None, *, skip_small_kv=False, attn_func=None):
+        super().__init__()
+        if _world_size(mesh) > 1:
+            raise NotImplementedError("this build runs on one GPU: ulysses / ring meshes of more than one rank are not provided")
+        self._parallel_method = "ulysses"
+        self._skip_small_kv = skip_small_kv
+        self._attn_func = attn_func
+
+    def __torch_function__(self, func, types, args=(), kwargs=None):
+        kwargs = {} if kwargs is None else kwargs
+        if UnifiedAttnMode.disabled:
+            return func(*args, **kwargs)
+        if func is F.scaled_dot_product_attention:
+            if self._skip_small_kv:
+                b = _bind(args, kwargs)
+                if b["query"].shape[-2] > b["key"].shape[-2]:
+                    return func(*args, **kwargs)
+            return self._call_unified_attn_func(*args, **kwargs)
+        return func(*args, **kwargs)
+
+    def _call_unified_attn_func(self, *args, **kwargs):
+        func = F.scaled_dot_product_attention
+        method = self._parallel_method
+        if method in ("ulysses", "ring"):  # world size 1: both stages pass the call on
+            self._parallel_method = "ring" if method == "ulysses" else "none"
+            try:
+                with self:
+                    return func(*args, **kwargs)
+            finally:
+                self._parallel_method = method
+        if method != "none":
+            raise ValueError(f"Unknown parallel method: {method}")
+        if config.attention.force_dispatch_to_custom_ops:
+            return ops.attention_forward(*args, **kwargs)
+        if self._attn_func is not None:
+            return self._attn_func(*args, **kwargs)
+        if kernel_takes(**_bind(args, kwargs)):
+            b = _bind(args, kwargs)
+            b.pop("enable_gqa", None)
+            return ops.attention_forward(**b)
+        return func(*args, **kwargs)
+
+    @classmethod
+    @contextlib.contextmanager
+    def disable(cls):
+        old = cls._set_disabled(True)
+        try:
+            yield
+        finally:
+            cls._set_disabled(old)
+
+    @classmethod
+    @torch.compiler.disable
+    def _set_disabled(cls, value):
+        old = cls.disabled
+        cls.disabled = value
+        return old
+
+
+def sparse_kv_attn_func(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None,
+                        dispatch_to_custom_ops=True):
+    """src/para_attn/sparse_attn.py:49-69: SDPA that drops the keys a boolean mask switches off.
+    Both settings of ``dispatch_to_custom_ops`` end in the same kernel here."""
+    return ops.attention_forward_sparse_kv(query, key, value, attn_mask=attn_mask, dropout_p=dropout_p,
+                                           is_causal=is_causal, scale=scale)
+
+
+class SparseKVAttnMode(TorchFunctionMode):
+    """src/para_attn/sparse_attn.py:607-640."""
+
+    disabled = False
+
+    @torch.compiler.disable
+    def __init__(self, *, dispatch_to_custom_ops=True):
+        super().__init__()
+        self._dispatch_to_custom_ops = dispatch_to_custom_ops
+
+    def __torch_function__(self, func, types, args=(), kwargs=None):
+        kwargs = {} if kwargs is None else kwargs
+        if SparseKVAttnMode.disabled:
+            return func(*args, **kwargs)
+        if func is F.scaled_dot_product_attention:
+            return sparse_kv_attn_func(*args, **kwargs, dispatch_to_custom_ops=self._dispatch_to_custom_ops)
+        return func(*args, **kwargs)
+
+    @classmethod
+    @contextlib.contextmanager
+    def disable(cls):
+        old = cls._set_disabled(True)
+        try:
+            yield
+        finally:
+            cls._set_disabled(old)
+
+    @classmethod
+    @torch.compiler.disable
+    def _set_disabled(cls, value):
+        old = cls.disabled
+        cls.disabled = value
+        return old

@@ -169,3 +169,40 @@ def test_taylorseer_schedule_and_limits():
     assert ts.approximate_value() == 0  # nothing stored: the reference's empty sum
     with pytest.raises(NotImplementedError):
         TaylorSeer(n_derivatives=5)
+
+
+def test_unified_attn_mode_on_cpu_passes_through():
+    """Calls the kernel does not take (CPU tensors here) reach F.scaled_dot_product_attention untouched, through
+    all three stages (para_attn_interface.py:445-475); a mesh of several ranks is refused."""
+    import torch
+    import torch.nn.functional as F
+
+    import paraattention_amd
+    from paraattention_amd import interface
+
+    q, k, v = (torch.randn(1, 2, 8, 16) for _ in range(3))
+    want = F.scaled_dot_product_attention(q, k, v)
+    with paraattention_amd.UnifiedAttnMode():
+        got = F.scaled_dot_product_attention(q, k, v)
+        assert torch.equal(torch.add(q, 1), q + 1)  # other functions are left alone
+    assert torch.equal(got, want)
+    calls = []
+    with paraattention_amd.UnifiedAttnMode(attn_func=lambda *a, **kw: calls.append((a, kw)) or "mine"):
+        assert F.scaled_dot_product_attention(q, k, v, scale=0.5) == "mine"
+    assert len(calls) == 1 and calls[0][1] == {"scale": 0.5}
+    with paraattention_amd.UnifiedAttnMode(skip_small_kv=True, attn_func=lambda *a, **kw: "mine"):
+        assert F.scaled_dot_product_attention(q, k[:, :, :4], v[:, :, :4]) is not "mine"  # more queries than keys: skipped
+        assert F.scaled_dot_product_attention(q[:, :, :4], k, v) == "mine"
+    with paraattention_amd.UnifiedAttnMode(attn_func=lambda *a, **kw: "mine"):
+        with paraattention_amd.UnifiedAttnMode.disable():
+            assert torch.equal(F.scaled_dot_product_attention(q, k, v), want)
+    assert not interface.kernel_takes(q, k, v)
+
+    class FakeMesh:
+        def size(self):
+            return 8
+
+    import pytest
+
+    with pytest.raises(NotImplementedError):
+        paraattention_amd.UnifiedAttnMode(FakeMesh())
