@@ -115,7 +115,7 @@ def test_permutation_invariance(cuda):
 
 
 def test_flux_shape_vs_torch_cpu(cuda):
-    # BASELINE config 1: B1 H24 S4608 D128 against torch's CPU SDPA on identical bits
+    # the FLUX-dev joint-attention shape: B1 H24 S4608 D128 against torch's CPU SDPA on identical bits
     q, k, v = inputs.qkv(1, 24, 4608, 4608, 128, seed=0)
     ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q, k, v)
     out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
@@ -123,7 +123,7 @@ def test_flux_shape_vs_torch_cpu(cuda):
 
 
 def test_hunyuan_shape_sampled_rows(cuda):
-    # BASELINE config 2 at full size on the GPU; the oracle checks sampled query rows of each head
+    # the 119k-token HunyuanVideo head-share shape at full size on the GPU; the oracle checks sampled query rows of each head
     B, H, S, D = 1, 3, 119056, 128
     q, k, v = inputs.qkv(B, H, S, S, D, seed=0, rms_norm_qk=True)
     out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
@@ -134,7 +134,7 @@ def test_hunyuan_shape_sampled_rows(cuda):
 
 
 def test_wan_cross_attention_shape(cuda):
-    # BASELINE config 4 cross-attention: 32760 queries x 512 text keys (reduced heads for the CPU check)
+    # the Wan 2.1 shape cross-attention: 32760 queries x 512 text keys (reduced heads for the CPU check)
     q, k, v = inputs.qkv(1, 4, 32760, 512, 128, seed=2)
     ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q, k, v)
     out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))

@@ -30,7 +30,7 @@ def test_ratio_bit_exact(cuda, shape, dtype, noise):
 
 
 def test_wan_shape_decision(cuda):
-    # BASELINE config 4: bf16 [1,32760,5120] pair, threshold 0.12 -> hit; 0.2 noise -> miss
+    # the Wan 2.1 shape: bf16 [1,32760,5120] pair, threshold 0.12 -> hit; 0.2 noise -> miss
     prev, cur = inputs.fbcache_pair((1, 32760, 5120), seed=1234, noise=0.05)
     want, md, mt = ofb.residual_diff_ratio(prev.float().numpy(), cur.float().numpy())
     got = torch.ops.para_attn.fbcache_residual_diff(prev.to(cuda), cur.to(cuda)).item()

@@ -75,7 +75,7 @@ def test_merge_empty_partials(cuda):
 
 @pytest.mark.parametrize("fused", [True, False])
 def test_ring_sweep_equals_full_attention(cuda, fused):
-    # BASELINE config 3 in miniature, ragged like 14882 = 116*128 + 34: 8 blocks of 290 keys
+    # the ring-sweep shape in miniature, ragged like 14882 = 116*128 + 34: 8 blocks of 290 keys
     B, H, Sq, D, nblk, blk = 1, 4, 290, 128, 8, 290
     q, k, v = inputs.qkv(B, H, Sq, nblk * blk, D, seed=3)
     ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
@@ -130,7 +130,7 @@ def test_fused_accumulate_steps(cuda, monkeypatch):
 
 
 def test_ring_sweep_full_shape_sampled(cuda):
-    # BASELINE config 3 at full size (Q block 14882 x 24 heads against 8 KV blocks of 14882);
+    # the ring-sweep shape at full size (Q block 14882 x 24 heads against 8 KV blocks of 14882);
     # the oracle checks sampled rows of two heads against one full-length SDPA over 119056 keys
     B, H, Sq, D, nblk = 1, 24, 14882, 128, 8
     g = torch.Generator().manual_seed(0)

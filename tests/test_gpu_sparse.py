@@ -114,7 +114,7 @@ def test_row_without_kept_block(cuda):
 
 
 def test_config5_shape_sampled(cuda):
-    # BASELINE config 5: B1 H24 S32768 D128, 128x128 tiles, ~30% density; the oracle checks sampled
+    # the block-sparse benchmark shape: B1 H24 S32768 D128, 128x128 tiles, ~30% density; the oracle checks sampled
     # query blocks of sampled heads by gathering their kept key blocks (torch CPU SDPA)
     B, H, S, D, nb = 1, 24, 32768, 128, 256
     q, k, v = inputs.qkv(B, H, S, S, D, seed=0)

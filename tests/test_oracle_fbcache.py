@@ -91,7 +91,7 @@ def test_decision_table():
 
 
 def test_wan_row_slice_known_answer():
-    """A 1/16 row slice of BASELINE config 4 (the full [1,32760,5120] pair is checked in the GPU suite,
+    """A 1/16 row slice of the Wan 2.1 shape (the full [1,32760,5120] pair is checked in the GPU suite,
     where the host has the memory bandwidth for it): torch's chain and the oracle agree to the bit."""
     prev, cur = inputs.fbcache_pair((1, 2048, 5120), seed=1234, noise=0.05)
     got = ofb.residual_diff_ratio(prev.float().numpy(), cur.float().numpy())
