@@ -47,9 +47,11 @@ PA_API int pa_abi_version(void);
 PA_API const char* pa_last_error(void);
 
 /*
- * Dense non-causal scaled-dot-product attention forward.
+ * Dense scaled-dot-product attention forward.
  *   out[b,h,i,:] = softmax_j(scale * q[b,h,i,:].k[b,h,j,:]) @ v[b,h,j,:]
  *   lse[b,h,i]   = log sum_j exp(scale * q.k)      (natural log, fp32)
+ * with j over all keys, or, with is_causal != 0, over keys j <= i (torch's
+ * is_causal: the lower-left triangle aligned at the top-left corner).
  * Stands in for para_attn.ops.attention_forward_with_lse
  * (src/para_attn/ops/__init__.py:112-179: the aten flash / efficient / cuDNN
  * forward + [:2]) and, with lse == NULL, for para_attn.ops.attention_forward
@@ -61,12 +63,13 @@ PA_API const char* pa_last_error(void);
  * kv_len: NULL, or int32 [B] device array giving, per batch element, how many
  * leading keys take part (the rest are ignored); this is how the sparse_kv op
  * (src/para_attn/ops/__init__.py:248-299) runs once its mask is a prefix.
+ * is_causal: the op's argument of the same name (ops/__init__.py:117, 138).
  */
 PA_API int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* out, float* lse,
                     int dtype, int B, int H, int Sq, int Skv, int D,
                     const int64_t q_strides[3], const int64_t k_strides[3],
                     const int64_t v_strides[3], const int64_t out_strides[3],
-                    float scale, const int32_t* kv_len, void* stream);
+                    float scale, const int32_t* kv_len, int is_causal, void* stream);
 
 /*
  * pa_attn_fwd_lse with a workspace lent by the caller.  The reference's op
@@ -85,7 +88,7 @@ PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void*
                        int dtype, int B, int H, int Sq, int Skv, int D,
                        const int64_t q_strides[3], const int64_t k_strides[3],
                        const int64_t v_strides[3], const int64_t out_strides[3],
-                       float scale, const int32_t* kv_len, void* workspace,
+                       float scale, const int32_t* kv_len, int is_causal, void* workspace,
                        size_t workspace_bytes, void* stream);
 
 /*

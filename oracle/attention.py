@@ -34,7 +34,14 @@ def sdpa_lse_f64(q, k, v, scale=None, keep=None):
     return out, lse
 
 
-def sdpa_lse_torch_cpu(q, k, v, scale=None, attn_mask=None):
+def causal_keep(Sq, Skv):
+    """torch's is_causal mask (what the aten kernels apply for
+    src/para_attn/ops/__init__.py:117, 138): query i keeps keys j <= i, the lower
+    triangle aligned at the top-left corner, for any Sq and Skv."""
+    return np.arange(Skv)[None, :] <= np.arange(Sq)[:, None]
+
+
+def sdpa_lse_torch_cpu(q, k, v, scale=None, attn_mask=None, is_causal=False):
     """torch's CPU flash kernel: the library routine the reference's SDPA path reduces
     to off-GPU (bit-equal to F.scaled_dot_product_attention on CPU).
 
@@ -47,6 +54,6 @@ def sdpa_lse_torch_cpu(q, k, v, scale=None, attn_mask=None):
     if mask is not None and mask.dtype == torch.bool:
         mask = torch.zeros(mask.shape, dtype=q.dtype).masked_fill_(~mask, float("-inf"))
     out, lse = torch.ops.aten._scaled_dot_product_flash_attention_for_cpu(
-        q, k, v, dropout_p=0.0, is_causal=False, attn_mask=mask, scale=scale
+        q, k, v, dropout_p=0.0, is_causal=is_causal, attn_mask=mask, scale=scale
     )
     return out, lse

@@ -22,7 +22,7 @@ PA_DTYPE_BF16 = 0
 PA_DTYPE_F16 = 1
 PA_DTYPE_F32 = 2
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -39,11 +39,11 @@ SIGNATURES = {
     "pa_last_error": (ctypes.c_char_p, []),
     "pa_attn_fwd_lse": (
         _i,
-        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _vp],
+        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _i, _vp],
     ),
     "pa_attn_fwd_lse_ws": (
         _i,
-        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp,
+        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _i,
          _vp, _sz, _vp],
     ),
     "pa_attn_fwd_accumulate": (

@@ -56,6 +56,7 @@ struct AttnParams {
   int bm;            // query rows per workgroup (32 per wavefront)
   int pipe;          // head_dim 128: 1 = pipelined kernel, 0 = the one without 32-bit offset limits
   const int32_t* kv_len;  // dense: optional per-batch key count
+  int causal;             // dense: query row i sees keys 0..i only (torch's is_causal, top-left aligned)
   // block-sparse only
   const int32_t* runs;  // count[Hm*nSeg] then range[Hm*nSeg][cap][2]
   int Hm, nQ, cap;
@@ -174,6 +175,8 @@ __device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int he
     const int cnt = p.runs[sidx];
     it.init_list(p.runs + (size_t)p.Hm * nseg + (size_t)sidx * p.cap * 2, cnt);
   } else {
+    // causal: a workgroup's work grows with its row index, so the longest ones are started first
+    if (p.causal) qt = p.n_qtiles - 1 - qt;
     row_begin = qt * p.bm;
     row_end = row_begin + p.bm < p.Sq ? row_begin + p.bm : p.Sq;
     int len = p.Skv;
@@ -181,6 +184,7 @@ __device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int he
       int kl = p.kv_len[batch];
       len = kl < len ? (kl < 0 ? 0 : kl) : len;
     }
+    if (p.causal && len > row_end) len = row_end;  // no row of this workgroup sees a key past its last row
     it.init_dense(len);
   }
 
@@ -330,6 +334,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     store_tile(0);
   }
   int cur_valid = nvalid;
+  int cur_n0 = 0;  // first key of the current tile (dense ranges start at key 0 and are contiguous)
+  const int wave_row0 = row_begin + 32 * (threadIdx.x >> 6);
   bool have_next = it.valid();
   int next_valid = 0;
   if (have_next) {
@@ -373,13 +379,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     }
 
     // ---- mask the ragged end of a range ---------------------------------------
-    if (cur_valid < BN) {
+    if (cur_valid < BN || (!SPARSE && p.causal && cur_n0 + BN - 1 > wave_row0)) {
+      int lim = cur_valid;
+      if (!SPARSE && p.causal) lim = min(lim, my_row - cur_n0 + 1);  // keys up to the row's own index
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           int n = 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
-          if (n >= cur_valid) s[t][r] = -INFINITY;
+          if (n >= lim) s[t][r] = -INFINITY;
         }
     }
 
@@ -432,6 +440,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     buf ^= 1;
     have = have_next;
     cur_valid = next_valid;
+    cur_n0 += BN;
     have_next = have_next2;
     next_valid = next2_valid;
   }
@@ -609,6 +618,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 
   // ---- prologue: K0, V0, K1 in flight; first K fragments in registers --------------------------
   int n0 = 0, cur_valid = 0, next_valid = 0;
+  int cur_n0 = 0;  // first key of the current tile (dense ranges start at key 0 and are contiguous)
+  const int wave_row0 = row_begin + 32 * wave;
   bool have = itK.valid();
   bool have_next = false;
   vec8 fa[8], fb[8];
@@ -666,12 +677,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 #pragma unroll
       for (int db = 0; db < DB; ++db) fa[cc * 4 + db] = read_vt(tV, 0, cc, db);
 
-    if (cur_valid < BN) {
+    if (cur_valid < BN || (!SPARSE && p.causal && cur_n0 + BN - 1 > wave_row0)) {
+      int lim = cur_valid;
+      if (!SPARSE && p.causal) lim = min(lim, my_row - cur_n0 + 1);  // keys up to the row's own index
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         int n = 8 * (r >> 2) + 4 * hh + (r & 3);
-        if (n >= cur_valid) s0[r] = -INFINITY;
-        if (n + 32 >= cur_valid) s1[r] = -INFINITY;
+        if (n >= lim) s0[r] = -INFINITY;
+        if (n + 32 >= lim) s1[r] = -INFINITY;
       }
     }
     float mx = fmaxf(s0[0], s0[1]);
@@ -746,6 +759,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 
     have = have_next;
     cur_valid = next_valid;
+    cur_n0 += BN;
     have_next = more_k;
     next_valid = k2_valid;
   };
@@ -962,8 +976,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   // -inf on the keys past the end of a ragged tile: register r of this lane is key
   // 8*(r/4) + r%4 + 4*hh of the first half (+32 for the second); constants against one per-lane
   // limit, so nothing per register stays live across the loop
-  auto mask_tail = [&](floatx16& a0, floatx16& a1, int nvalid) {
-    const int lim = nvalid - 4 * hh;
+  const int wave_row0 = row_begin + 32 * wave;
+  // causal: the tile starting at key n0 needs masking for this wavefront if it reaches past its first row
+  auto on_diagonal = [&](uint32_t n0) {
+    if constexpr (SPARSE) return false;
+    else return p.causal != 0 && n0 != OOB && (int)n0 + BN - 1 > wave_row0;
+  };
+  auto mask_tail = [&](floatx16& a0, floatx16& a1, int nvalid, uint32_t n0) {
+    int lim = nvalid;
+    if constexpr (!SPARSE) {
+      if (p.causal) lim = min(lim, my_row - (int)n0 + 1);  // keys up to the row's own index
+    }
+    lim -= 4 * hh;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       if (8 * (r >> 2) + (r & 3) >= lim) a0[r] = -INFINITY;
@@ -1001,7 +1025,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     }
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
-    if (v_cur < BN) mask_tail(sn0, sn1, v_cur);
+    if (v_cur < BN || on_diagonal(n_cur)) mask_tail(sn0, sn1, v_cur, n_cur);
     float m2 = fmaxf(sn0[0], sn1[0]);
 #pragma unroll
     for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
@@ -1085,7 +1109,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       if (g < 4) expo_slot(8 + g);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (v_nxt < BN) mask_tail(sn0, sn1, v_nxt);  // ragged (or absent) tile j+1
+    if (v_nxt < BN || on_diagonal(n_nxt)) mask_tail(sn0, sn1, v_nxt, n_nxt);  // ragged, absent or diagonal tile j+1
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage B ---------------------------------------------------------------------------------
@@ -1401,6 +1425,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.tiles_left = 0; p.tiles_per_block = 0;
   p.bm = BM; p.pipe = 0;
   p.xcd_chunk = 0;
+  p.causal = 0;
   p.acc_out = nullptr; p.acc_lse = nullptr; p.acc_first = 0;
   p.split_main = 0; p.split_tiles = 0; p.split_s = 0; p.ws_out = nullptr; p.ws_lse = nullptr;
 }
@@ -1530,7 +1555,8 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
     return finish();
   }
   const int cus = device_cus();
-  const bool allow = cus > 0 && !env_is("PARAATTN_NO_SPLIT", "1") && (ws_needed != nullptr || ws_bytes > 0);
+  // (causal workgroups differ in length: the rounds estimate does not apply, no split)
+  const bool allow = cus > 0 && !p.causal && !env_is("PARAATTN_NO_SPLIT", "1") && (ws_needed != nullptr || ws_bytes > 0);
   const int kv_tiles = (p.Skv + BN - 1) / BN;
   const int64_t bh = (int64_t)p.B * p.H;
   const int64_t n128 = bh * ((p.Sq + 127) / 128), n256 = bh * ((p.Sq + 255) / 256);
@@ -1574,8 +1600,8 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
                           int dtype, int B, int H, int Sq, int Skv, int D,
                           const int64_t q_strides[3], const int64_t k_strides[3],
                           const int64_t v_strides[3], const int64_t out_strides[3], float scale,
-                          const int32_t* kv_len, void* workspace, size_t workspace_bytes, void* stream,
-                          float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0) {
+                          const int32_t* kv_len, int is_causal, void* workspace, size_t workspace_bytes,
+                          void* stream, float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0) {
   const int64_t zero3[3] = {0, 0, 0};
   const bool accumulate = acc_out != nullptr;
   if (accumulate) {
@@ -1590,8 +1616,10 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   AttnParams p;
   fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
   p.kv_len = kv_len;
+  p.causal = is_causal != 0;
   choose_kernel(p, D, 256, true, workspace ? workspace_bytes : 0, nullptr);
   if (accumulate) {
+    if (p.causal) PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation is not causal");
     if (!p.pipe)
       PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation needs head_dim 128 and K/V below 4 GiB per head; run pa_attn_fwd_lse and pa_merge_lse");
     p.acc_out = acc_out; p.acc_lse = acc_lse; p.acc_first = acc_first != 0;
@@ -1608,19 +1636,19 @@ extern "C" int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void
                                int dtype, int B, int H, int Sq, int Skv, int D,
                                const int64_t q_strides[3], const int64_t k_strides[3],
                                const int64_t v_strides[3], const int64_t out_strides[3],
-                               float scale, const int32_t* kv_len, void* stream) {
+                               float scale, const int32_t* kv_len, int is_causal, void* stream) {
   return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
-                        out_strides, scale, kv_len, nullptr, 0, stream);
+                        out_strides, scale, kv_len, is_causal, nullptr, 0, stream);
 }
 
 extern "C" int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void* out, float* lse,
                                   int dtype, int B, int H, int Sq, int Skv, int D,
                                   const int64_t q_strides[3], const int64_t k_strides[3],
                                   const int64_t v_strides[3], const int64_t out_strides[3],
-                                  float scale, const int32_t* kv_len, void* workspace,
+                                  float scale, const int32_t* kv_len, int is_causal, void* workspace,
                                   size_t workspace_bytes, void* stream) {
   return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
-                        out_strides, scale, kv_len, workspace, workspace_bytes, stream);
+                        out_strides, scale, kv_len, is_causal, workspace, workspace_bytes, stream);
 }
 
 extern "C" int pa_attn_fwd_accumulate(const void* q, const void* k, const void* v, float* acc_out,
@@ -1633,7 +1661,7 @@ extern "C" int pa_attn_fwd_accumulate(const void* q, const void* k, const void* 
   if (!acc_out || !acc_lse) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
   if (out && !out_strides) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
   return attn_fwd_dense(q, k, v, out, nullptr, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
-                        out_strides, scale, kv_len, workspace, workspace_bytes, stream, acc_out, acc_lse, first);
+                        out_strides, scale, kv_len, 0, workspace, workspace_bytes, stream, acc_out, acc_lse, first);
 }
 
 extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,

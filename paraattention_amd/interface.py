@@ -32,7 +32,9 @@ def kernel_takes(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=Fal
         return False
     if query.dtype not in (torch.bfloat16, torch.float16) or key.dtype != query.dtype or value.dtype != query.dtype:
         return False
-    if dropout_p != 0.0 or is_causal or enable_gqa or query.shape[1] != key.shape[1]:
+    if dropout_p != 0.0 or enable_gqa or query.shape[1] != key.shape[1]:
+        return False
+    if is_causal and attn_mask is not None:
         return False
     if query.shape[-1] not in (64, 128) or value.shape[-1] != query.shape[-1]:
         return False

@@ -47,13 +47,15 @@ def _kernel_ready(t):
     return t
 
 
-def _check_sdpa_args(query, key, value, dropout_p, is_causal):
+def _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask=None, causal_ok=False):
     if query.ndim != 4 or key.ndim != 4 or value.ndim != 4:
         raise ValueError("query, key and value must be 4-D [batch, heads, seq, head_dim]")
     if dropout_p != 0.0:
         raise NotImplementedError("dropout_p > 0 is not supported (the reference's hot path is inference only)")
-    if is_causal:
-        raise NotImplementedError("is_causal=True is not supported by the gfx950 attention kernel")
+    if is_causal and not causal_ok:
+        raise NotImplementedError("is_causal=True is not supported by this op")
+    if is_causal and attn_mask is not None:
+        raise ValueError("an explicit attn_mask must not be set when is_causal=True")  # as torch's SDPA
     if query.dtype not in (torch.bfloat16, torch.float16):
         raise NotImplementedError(f"attention dtype {query.dtype} not supported (bf16 / fp16)")
     if key.dtype != query.dtype or value.dtype != query.dtype:
@@ -85,7 +87,7 @@ def _key_keep_vector(attn_mask, B, Skv):
     return m.expand(B, Skv)
 
 
-def _dense_forward(query, key, value, scale, want_lse, kv_len=None):
+def _dense_forward(query, key, value, scale, want_lse, kv_len=None, is_causal=False):
     B, H, Sq, D = query.shape
     Skv = key.shape[2]
     q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
@@ -105,7 +107,7 @@ def _dense_forward(query, key, value, scale, want_lse, kv_len=None):
         rc = lib.pa_attn_fwd_lse_ws(
             _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
             _lib.strides3(q), ks, vs, _lib.strides3(out),
-            float(scale), _ptr(kv_len), _ptr(ws), ws_bytes, _stream_ptr(q.device),
+            float(scale), _ptr(kv_len), 1 if is_causal else 0, _ptr(ws), ws_bytes, _stream_ptr(q.device),
         )
     _lib.check(rc, "pa_attn_fwd_lse_ws")
     return out, lse
@@ -139,10 +141,10 @@ def _accumulate_forward(acc_out, acc_lse, query, key, value, scale, first, final
     return out
 
 
-def _masked_forward(query, key, value, attn_mask, scale, want_lse):
-    """attn_mask handling shared by the three SDPA-signature ops."""
+def _masked_forward(query, key, value, attn_mask, scale, want_lse, is_causal=False):
+    """attn_mask / is_causal handling shared by the three SDPA-signature ops."""
     if attn_mask is None:
-        return _dense_forward(query, key, value, scale, want_lse)
+        return _dense_forward(query, key, value, scale, want_lse, is_causal=is_causal)
     B, Skv = query.shape[0], key.shape[2]
     keep = _key_keep_vector(attn_mask, B, Skv)
     if keep is None:
@@ -177,8 +179,8 @@ def attention_forward_with_lse(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """out [B,H,Sq,D] in query's dtype and natural-log LSE [B,H,Sq] in fp32
     (src/para_attn/ops/__init__.py:160-179)."""
-    _check_sdpa_args(query, key, value, dropout_p, is_causal)
-    out, lse = _masked_forward(query, key, value, attn_mask, scale, True)
+    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask, causal_ok=True)
+    out, lse = _masked_forward(query, key, value, attn_mask, scale, True, is_causal)
     return out, lse
 
 
@@ -202,8 +204,8 @@ def attention_forward(
     scale: Optional[float] = None,
 ) -> torch.Tensor:
     """Plain SDPA forward, no LSE (src/para_attn/ops/__init__.py:204-223)."""
-    _check_sdpa_args(query, key, value, dropout_p, is_causal)
-    out, _ = _masked_forward(query, key, value, attn_mask, scale, False)
+    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask, causal_ok=True)
+    out, _ = _masked_forward(query, key, value, attn_mask, scale, False, is_causal)
     return out
 
 

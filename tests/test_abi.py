@@ -57,17 +57,17 @@ def test_argument_validation_without_device_work():
     a = ctypes.c_void_p(base)
     st = (ctypes.c_int64 * 3)(0, 4096, 128)
     # unsupported head_dim, dtype, scale, misalignment
-    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 1, 1, 16, 16, 32, st, st, st, st, 1.0, None, None) == _lib.PA_ERR_UNSUPPORTED
+    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 1, 1, 16, 16, 32, st, st, st, st, 1.0, None, 0, None) == _lib.PA_ERR_UNSUPPORTED
     assert b"head_dim" in lib.pa_last_error()
-    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 2, 1, 1, 16, 16, 128, st, st, st, st, 1.0, None, None) == _lib.PA_ERR_UNSUPPORTED
-    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 1, 1, 16, 16, 128, st, st, st, st, -1.0, None, None) == _lib.PA_ERR_UNSUPPORTED
+    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 2, 1, 1, 16, 16, 128, st, st, st, st, 1.0, None, 0, None) == _lib.PA_ERR_UNSUPPORTED
+    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 1, 1, 16, 16, 128, st, st, st, st, -1.0, None, 0, None) == _lib.PA_ERR_UNSUPPORTED
     odd = ctypes.c_void_p(base + 2)
-    assert lib.pa_attn_fwd_lse(odd, a, a, a, None, 0, 1, 1, 16, 16, 128, st, st, st, st, 1.0, None, None) == _lib.PA_ERR_UNSUPPORTED
+    assert lib.pa_attn_fwd_lse(odd, a, a, a, None, 0, 1, 1, 16, 16, 128, st, st, st, st, 1.0, None, 0, None) == _lib.PA_ERR_UNSUPPORTED
     bad = (ctypes.c_int64 * 3)(0, 4096, 100)
-    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 1, 1, 16, 16, 128, bad, st, st, st, 1.0, None, None) == _lib.PA_ERR_UNSUPPORTED
-    assert lib.pa_attn_fwd_lse(None, a, a, a, None, 0, 1, 1, 16, 16, 128, st, st, st, st, 1.0, None, None) == _lib.PA_ERR_INVALID
+    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 1, 1, 16, 16, 128, bad, st, st, st, 1.0, None, 0, None) == _lib.PA_ERR_UNSUPPORTED
+    assert lib.pa_attn_fwd_lse(None, a, a, a, None, 0, 1, 1, 16, 16, 128, st, st, st, st, 1.0, None, 0, None) == _lib.PA_ERR_INVALID
     # empty problems succeed without touching the device
-    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 0, 1, 16, 16, 128, st, st, st, st, 1.0, None, None) == _lib.PA_OK
+    assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 0, 1, 16, 16, 128, st, st, st, st, 1.0, None, 0, None) == _lib.PA_OK
     assert lib.pa_merge_lse(a, 2, a, a, 0, a, a, 2, a, 0, 128, None) == _lib.PA_OK
     # merge: head_dim must be a multiple of 8; in-place needs equal dtypes
     assert lib.pa_merge_lse(a, 2, a, a, 0, a, a, 2, a, 4, 12, None) == _lib.PA_ERR_UNSUPPORTED

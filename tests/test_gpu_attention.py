@@ -212,7 +212,7 @@ def test_key_split_tail(cuda, bm, monkeypatch):
     short = torch.empty(64, dtype=torch.uint8, device=cuda)
     vp = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
     rc = lib.pa_attn_fwd_lse_ws(vp(qd), vp(kd), vp(vd), vp(out3), vp(lse3), 0, B, H, Sq, Skv, D, _lib.strides3(qd),
-                                _lib.strides3(kd), _lib.strides3(vd), _lib.strides3(out3), 1.0 / math.sqrt(D), None,
+                                _lib.strides3(kd), _lib.strides3(vd), _lib.strides3(out3), 1.0 / math.sqrt(D), None, 0,
                                 vp(short), short.numel(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     assert rc == 0
     torch.cuda.synchronize()
@@ -229,6 +229,59 @@ def test_key_split_tail(cuda, bm, monkeypatch):
     out2, lse2 = torch.ops.para_attn.attention_forward_with_lse(qs, kd, vd, keep[:, None, None, :].to(cuda))
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
     monkeypatch.delenv("PARAATTN_BM")
+
+
+CAUSAL = [(1, 2, 1, 1), (1, 1, 17, 17), (2, 2, 64, 64), (1, 2, 129, 129), (1, 1, 300, 300), (1, 2, 700, 700),
+          (1, 1, 300, 90), (1, 2, 90, 300), (1, 1, 1000, 1000)]
+
+
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("B,H,Sq,Skv", CAUSAL)
+def test_causal_vs_f64(cuda, B, H, Sq, Skv, D):
+    """is_causal=True as the reference's own op test asks for it (tests/ops/test_ops.py:28-31), plus Sq != Skv with
+    torch's top-left alignment.  Every kernel variant must agree with the oracle."""
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=Sq * 7 + Skv)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, oattn.causal_keep(Sq, Skv))
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, is_causal=True)
+    _check(out, lse, ref_out, ref_lse, f"causal {(B, H, Sq, Skv, D)}")
+    assert torch.equal(torch.ops.para_attn.attention_forward(qd, kd, vd, is_causal=True), out)
+
+
+@pytest.mark.parametrize("env", [{"PARAATTN_NO_PIPE": "1"}, {"PARAATTN_BM": "256"}, {"PARAATTN_BM": "128"}])
+def test_causal_alternative_kernels(cuda, env, monkeypatch):
+    for B, H, Sq, Skv in [(1, 2, 700, 700), (1, 1, 300, 90), (1, 2, 90, 300), (2, 1, 513, 513)]:
+        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=Sq + Skv)
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, oattn.causal_keep(Sq, Skv))
+        for name, val in env.items():
+            monkeypatch.setenv(name, val)
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), is_causal=True)
+        for name in env:
+            monkeypatch.delenv(name)
+        _check(out, lse, ref_out, ref_lse, f"causal {env} {(B, H, Sq, Skv)}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_causal_reference_test_shape(cuda, dtype, D):
+    """The reference's op test shape (tests/ops/test_ops.py:21-31: B1 H24 S4096, fp16 and bf16, is_causal) against
+    torch's CPU SDPA with is_causal, on a subset of heads."""
+    B, H, S = 1, 24, 4096
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=3, dtype=dtype)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), is_causal=True)
+    assert lse.dtype == torch.float32 and lse.shape == (B, H, S)
+    hs = [0, 11, 23]
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, hs].float(), k[:, hs].float(), v[:, hs].float(), is_causal=True)
+    _check(out[:, hs], lse[:, hs], ref_out.numpy(), ref_lse.numpy(), f"causal 4096 {dtype} D={D}")
+
+
+def test_causal_argument_rules(cuda):
+    q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 32, 32, 128))
+    mask = torch.ones(1, 1, 1, 32, dtype=torch.bool, device=cuda)
+    with pytest.raises(ValueError):
+        torch.ops.para_attn.attention_forward_with_lse(q, k, v, mask, is_causal=True)
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward_sparse_kv(q, k, v, mask, is_causal=True)
 
 
 def test_key_rows_spread_over_4gib(cuda):
@@ -255,8 +308,6 @@ def test_key_rows_spread_over_4gib(cuda):
 
 def test_unsupported_raise(cuda):
     q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 128))
-    with pytest.raises(NotImplementedError):
-        torch.ops.para_attn.attention_forward_with_lse(q, k, v, is_causal=True)
     with pytest.raises(NotImplementedError):
         torch.ops.para_attn.attention_forward_with_lse(q, k, v, dropout_p=0.1)
     with pytest.raises(NotImplementedError):

@@ -122,3 +122,21 @@ def test_matches_torch_cpu_sdpa(shape, dtype):
     o64m, l64m = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, keep.numpy())
     np.testing.assert_allclose(om.float().numpy(), o64m, atol=2e-2, rtol=2e-2)
     np.testing.assert_allclose(lm.numpy(), l64m, atol=1e-3)
+
+
+@pytest.mark.parametrize("Sq,Skv", [(1, 1), (5, 5), (7, 3), (3, 7), (70, 70), (33, 100), (100, 33)])
+def test_causal_keep_matches_torch(Sq, Skv):
+    """The causal mask: by its definition on tiny cases (row i keeps exactly min(i + 1, Skv) leading keys), against
+    torch's own is_causal (CPU SDPA) and against torch's documented construction ones(L, S).tril()."""
+    keep = oattn.causal_keep(Sq, Skv)
+    assert keep.shape == (Sq, Skv)
+    for i in range(Sq):
+        n = min(i + 1, Skv)
+        assert keep[i, :n].all() and not keep[i, n:].any()
+    assert np.array_equal(keep, torch.ones(Sq, Skv, dtype=torch.bool).tril(diagonal=0).numpy())
+    g = torch.Generator().manual_seed(Sq * 100 + Skv)
+    q, k, v = torch.randn(1, 2, Sq, 32, generator=g), torch.randn(1, 2, Skv, 32, generator=g), torch.randn(1, 2, Skv, 32, generator=g)
+    out, lse = oattn.sdpa_lse_f64(q.numpy(), k.numpy(), v.numpy(), None, keep)
+    t_out, t_lse = oattn.sdpa_lse_torch_cpu(q, k, v, is_causal=True)
+    np.testing.assert_allclose(out, t_out.numpy(), atol=2e-5, rtol=2e-5)
+    np.testing.assert_allclose(lse, t_lse.numpy(), atol=2e-5, rtol=2e-5)
