@@ -55,3 +55,38 @@ def test_sparse_kv_mode(cuda):
     with paraattention_amd.UnifiedAttnMode():
         out2 = F.scaled_dot_product_attention(q.to(cuda), k.to(cuda), v.to(cuda), attn_mask=keep[:, None, None, :].to(cuda))
     assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_compiled_function_under_the_mode(cuda, is_causal):
+    """The reference's mode test compiled (tests/test_interface.py:94-109): F.scaled_dot_product_attention inside
+    torch.compile(fullgraph=True), the mode entered around the call, two calls."""
+    q, k, v = (t.to(cuda) for t in inputs.qkv(1, 3, 257, 257, 128, seed=4))
+
+    def func(*args, **kwargs):
+        return F.scaled_dot_product_attention(*args, **kwargs)
+
+    compiled = torch.compile(func, fullgraph=True, backend="aot_eager")
+    for _ in range(2):
+        with paraattention_amd.UnifiedAttnMode():
+            out = compiled(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=is_causal)
+    assert torch.equal(out, torch.ops.para_attn.attention_forward(q, k, v, is_causal=is_causal))
+    keep = oattn.causal_keep(257, 257) if is_causal else None
+    ref_out, _ = oattn.sdpa_lse_f64(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), None, keep)
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+
+
+def test_compiled_ops_fullgraph(cuda):
+    """attention + merge custom ops inside one compiled graph (src/para_attn/ops/__init__.py registers them for this)."""
+    q, k, v = (t.to(cuda) for t in inputs.qkv(1, 2, 300, 200, 128, seed=5))
+
+    def fn(q, k, v):
+        o1, l1 = torch.ops.para_attn.attention_forward_with_lse(q, k[:, :, :120], v[:, :, :120])
+        o2, l2 = torch.ops.para_attn.attention_forward_with_lse(q, k[:, :, 120:], v[:, :, 120:])
+        return torch.ops.para_attn.merge_attention_lse(o1, l1, o2, l2, q.dtype)
+
+    want = fn(q, k, v)
+    got = torch.compile(fn, fullgraph=True, backend="aot_eager")(q, k, v)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    full, lse = torch.ops.para_attn.attention_forward_with_lse(q, k, v)
+    assert (got[0].float() - full.float()).abs().max().item() <= 2e-2 and (got[1] - lse).abs().max().item() <= 1e-3
