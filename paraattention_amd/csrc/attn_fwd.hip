@@ -1,8 +1,11 @@
-// Non-causal attention forward (output + fp32 log-sum-exp) for gfx950.
+// Attention forward (output + fp32 log-sum-exp, optionally causal) for gfx950.
 //
-// One workgroup = 4 wavefronts = 128 query rows; each wavefront owns 32 query
-// rows for the whole key sweep.  Keys/values stream through LDS in tiles of 64
-// rows, double buffered (global -> registers one tile ahead -> LDS).
+// One workgroup = 4 or 8 wavefronts = 128 or 256 query rows; each wavefront owns
+// 32 query rows for the whole key sweep.  Keys/values stream through LDS in
+// tiles of 64 rows, double buffered.  Three kernels share the scheme:
+//   attn_fwd_kernel            any head_dim (used for 64): global -> registers -> LDS
+//   attn_fwd_d128_kernel       head_dim 128, LDS-DMA fills, 64-bit addressing
+//   attn_fwd_d128_pipe_kernel  head_dim 128, two-tile software pipeline (the default)
 //
 // Both GEMMs run transposed so that the softmax needs no cross-lane traffic and
 // P never leaves registers:
@@ -806,13 +809,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 //
 //   barrier            K(j+1) and V(j) have landed; everybody is done with iteration j-1
 //   rare rescale of O  from the row maximum of S(j), taken one iteration earlier
-//   stage A  16 x { MFMA of S(j+1) = K(j+1) Q^T ; one LDS-DMA issue for K(j+2) / V(j+1) (first 8) ;
-//                   refill of the consumed fragment slot ; exp2 / sum / pack of two scores of S(j) }
-//   stage B  16 x { MFMA of O^T += V(j)^T P(j)^T ; refill ; part of the row maximum of S(j+1) }
+//   stage A  16 x { MFMA of S(j+1) = K(j+1) Q^T, its two key halves alternating ; one LDS-DMA issue
+//                   for K(j+2) / V(j+1) (first groups) ; refill of the consumed fragment slot ;
+//                   one slot of the softmax of S(j): scale, exp2, sum + pack of a score pair take
+//                   three consecutive slots }
+//   stage B  16 x { MFMA of O^T += V(j)^T P(j)^T ; refill ; the last softmax slots ; the row
+//                   maximum of S(j+1) }
 //
 // so exponentials, the issue stalls of the tile copies and the row maximum all sit in the shadow
 // of MFMAs of the same wavefront.  Every iteration runs the same code: a tile that does not exist
 // is fetched out of bounds (the buffer descriptor returns zeros) and its scores are never used.
+// NW = 4 wavefronts (128 query rows, two workgroups per CU) or 8 (256 rows, one per CU: half the
+// tile copies per flop).  Dense launches may compute the query tiles of the last round of
+// workgroups in several key shares (AttnParams::split_*), fold the result into a running
+// (out, lse) pair (acc_*), or apply torch's causal mask (causal).
 // ---------------------------------------------------------------------------------------------
 template <typename T, bool SPARSE, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_kernel(const AttnParams p) {
