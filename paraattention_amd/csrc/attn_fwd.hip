@@ -1459,11 +1459,13 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     smem = Smem<D>::BYTES;
     slot = 0;
   }
-  static bool attr_done[3] = {false, false, false};  // benign race: the call is idempotent
-  if (!attr_done[slot]) {
+  // the attribute belongs to the function on one device: remembered per device and kernel variant
+  static bool attr_done[PA_MAX_DEVICES][3] = {};  // benign race: the call is idempotent
+  const int dev = current_device();
+  if (dev < 0 || !attr_done[dev][slot]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_done[slot] = true;
+    if (dev >= 0) attr_done[dev][slot] = true;
   }
   if constexpr (D == 128) {
     if (slot == 2)
@@ -1484,19 +1486,6 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     }
   }
   return PA_OK;
-}
-
-// Compute units of the current device (0 if it cannot be asked), cached per device.
-static int device_cus() {
-  static int cus[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (cus[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-    cus[dev] = n;  // benign race: every thread writes the same value
-  }
-  return cus[dev];
 }
 
 // Key-split tail.  All workgroups of the dense kernel cost the same, so a grid of n_tiles

@@ -306,15 +306,8 @@ __global__ __launch_bounds__(FB_THREADS) void fbcache_apply_kernel(const void* r
 static inline int fb_grid(int64_t work_items, int per_cu = 1) {
   int64_t blocks = (work_items + FB_THREADS - 1) / FB_THREADS;
   if (blocks < 1) blocks = 1;
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      n_cu = v;
-    else
-      n_cu = 256;
-  }
+  int n_cu = device_cus();
+  if (n_cu <= 0) n_cu = 256;
   const int64_t cap = (int64_t)n_cu * per_cu;
   return (int)(blocks < cap ? blocks : cap);
 }

@@ -24,6 +24,29 @@ char* error_slot();  // 512-byte thread-local buffer (defined in pa_api.hip)
     if (e_ != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e_)); \
   } while (0)
 
+// ---- per-device facts --------------------------------------------------------
+constexpr int PA_MAX_DEVICES = 64;
+
+// Index of the current device, or -1 if it cannot be asked or is beyond the cached range.
+static inline int current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= PA_MAX_DEVICES) return -1;
+  return dev;
+}
+
+// Compute units of the current device (0 if it cannot be asked), cached per device.
+static inline int device_cus() {
+  static int cus[PA_MAX_DEVICES] = {0};
+  const int dev = current_device();
+  if (dev < 0) return 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cus[dev] = n;  // benign race: every thread writes the same value
+  }
+  return cus[dev];
+}
+
 // ---- vector types ---------------------------------------------------------
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
