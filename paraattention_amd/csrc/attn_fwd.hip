@@ -3,9 +3,10 @@
 // One workgroup = 4 or 8 wavefronts = 128 or 256 query rows; each wavefront owns
 // 32 query rows for the whole key sweep.  Keys/values stream through LDS in
 // tiles of 64 rows, double buffered.  Three kernels share the scheme:
-//   attn_fwd_kernel            any head_dim (used for 64): global -> registers -> LDS
+//   attn_fwd_kernel            any head_dim (64 when K or V spans 4 GiB or more): global -> registers -> LDS
 //   attn_fwd_d128_kernel       head_dim 128, LDS-DMA fills, 64-bit addressing
 //   attn_fwd_d128_pipe_kernel  head_dim 128, two-tile software pipeline (the default)
+//   attn_fwd_d64_pipe_kernel   head_dim 64, the same pipeline (the default)
 //
 // Both GEMMs run transposed so that the softmax needs no cross-lane traffic and
 // P never leaves registers:
@@ -1253,6 +1254,335 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// head_dim 64 (the reference's own op-test shape, tests/ops/test_ops.py:21-24): the two-tile
+// pipeline above with half the contraction and half the output width.  A K or V tile is 64 rows of
+// 128 bytes; one copy instruction moves 8 rows.  Swizzles for 128-byte rows (two rows share the 64
+// banks): K chunk c of row r sits at c ^ ((r >> 1) & 7), so the 16 rows a b128 read touches hit 16
+// different 16-byte slots; V chunk c at c ^ (4 * ((r >> 1) & 1)), so the two even (odd) rows of a
+// transpose read keep apart.  Per tile and wavefront: 8 MFMAs of S(j+1) (stage A), 8 of
+// O^T += V(j)^T P(j)^T (stage B), against the same 32 exponentials per lane as at head_dim 128, so
+// this kernel is bound by the VALU, not by the matrix cores.  The 8 fragments of K(j+1) fill the
+// ring at the top of an iteration; each stage-A MFMA frees a slot for one of the 8 fragments of
+// V(j); the 18 softmax slots sit two per group where the P half is needed soonest.
+// ---------------------------------------------------------------------------------------------
+constexpr int TILE64_BYTES = BN * 128;
+
+template <typename T, bool SPARSE, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_kernel(const AttnParams p) {
+  typedef typename T::vec8 vec8;
+  constexpr int DC = 4, DB = 2;
+  constexpr int IPW = 8 / NW;  // copy instructions per wavefront and K (V) tile
+  constexpr int RS = 8 * NW;   // tile rows between two of them
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  char* const sK = (char*)smem;                      // [2][64][128 B]
+  char* const sV = (char*)smem + 2 * TILE64_BYTES;   // [2][64][128 B]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  int tile = blockIdx.x;
+  if constexpr (SPARSE) {
+    if (p.xcd_chunk > 0) {  // one contiguous eighth of the (head, query tile) list per XCD
+      tile = (tile & 7) * p.xcd_chunk + (tile >> 3);
+      if (tile >= p.B * p.H * p.n_qtiles) return;
+    }
+  }
+  const int qt = tile % p.n_qtiles;
+  const int bh = tile / p.n_qtiles;
+  const int head = bh % p.H;
+  const int batch = bh / p.H;
+  int row_begin, row_end;
+  TileIter it;
+  decode_block<SPARSE>(p, qt, head, batch, row_begin, row_end, it);
+
+  const uint16_t* qbase = (const uint16_t*)p.q + batch * p.qs_b + head * p.qs_h;
+  const char* kbytes = (const char*)((const uint16_t*)p.k + batch * p.ks_b + head * p.ks_h);
+  const char* vbytes = (const char*)((const uint16_t*)p.v + batch * p.vs_b + head * p.vs_h);
+  const uint32_t ks_bytes = (uint32_t)(p.ks_s * 2), vs_bytes = (uint32_t)(p.vs_s * 2);
+
+  const int my_row = row_begin + wave * 32 + l32;
+  const bool row_ok = my_row < row_end;
+  vec8 qf[DC];
+  {
+    int r = row_ok ? my_row : (row_end - 1);
+    const uint16_t* qp = qbase + (int64_t)r * p.qs_s + 8 * hh;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): keep Q out of the loop's wait accounting
+  }
+
+  // global -> LDS copies as in the head_dim-128 pipeline: wave w, step i covers tile rows
+  // RS*i + 8w .. +7; lane l lands on chunk l%8 of row l/8
+  auto make_rsrc = [&](const char* base, uint32_t row_bytes) {
+    u32x4 r;
+    const uint64_t a = (uint64_t)base;
+    const uint64_t nbytes = (uint64_t)(p.Skv - 1) * row_bytes + 128;  // start of the last row + one row
+    r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+    r[2] = __builtin_amdgcn_readfirstlane((uint32_t)nbytes);
+    r[3] = 0x00020000u;
+    return r;
+  };
+  const u32x4 krs = make_rsrc(kbytes, ks_bytes);
+  const u32x4 vrs = make_rsrc(vbytes, vs_bytes);
+  const int dma_row = 8 * wave + (lane >> 3);
+  const int dma_pc = lane & 7;
+  const uint32_t k_off0 = dma_row * ks_bytes + 16 * (dma_pc ^ ((dma_row >> 1) & 7));
+  const uint32_t v_off0 = dma_row * vs_bytes + 16 * (dma_pc ^ (4 * ((dma_row >> 1) & 1)));
+  const uint32_t lds_k = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sK + wave * 1024);
+  const uint32_t lds_v = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sV + wave * 1024);
+  constexpr uint32_t OOB = PIPE_OOB;
+  auto dma_k1 = [&](int buf, uint32_t n0, int i) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * ks_bytes);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_k + buf * TILE64_BYTES + i * (RS * 128)), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
+  };
+  auto dma_v1 = [&](int buf, uint32_t n0, int i) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * vs_bytes);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_v + buf * TILE64_BYTES + i * (RS * 128)), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
+  };
+
+  // fragment read addresses
+  uint32_t ka[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) ka[dc] = l32 * 128 + 16 * ((2 * dc + hh) ^ ((l32 >> 1) & 7));
+  uint32_t va[DB];
+  {
+    const int g16 = lane >> 4, lg = lane & 15, r = lg >> 2, cq = lg & 3, dhalf = g16 & 1;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      va[db] = (4 * hh + r) * 128 + 16 * ((4 * db + 2 * dhalf + (cq >> 1)) ^ (4 * ((r >> 1) & 1))) + 8 * (cq & 1);
+  }
+  auto read_k = [&](const char* tl, int t, int dc) -> vec8 { return *(const vec8*)(tl + t * 32 * 128 + ka[dc]); };
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  auto read_vt = [&](const char* tl, int t, int c, int db) -> vec8 {
+    const char* a = tl + (32 * t + 16 * c) * 128 + va[db];
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + 8 * 128));
+    typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
+    s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(vec8, v);
+  };
+
+  floatx16 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale_log2;
+
+  uint32_t n_cur, n_nxt, n_nx2;
+  int v_cur, v_nxt, v_nx2;
+  auto pull = [&](uint32_t& n0, int& nv) {
+    if (it.valid()) {
+      int a, b;
+      it.get(a, b);
+      it.next();
+      n0 = (uint32_t)a;
+      nv = b;
+    } else {
+      n0 = OOB;
+      nv = 0;
+    }
+  };
+  pull(n_cur, v_cur);
+  pull(n_nxt, v_nxt);
+  pull(n_nx2, v_nx2);
+  bool have = n_cur != OOB;
+
+  const int wave_row0 = row_begin + 32 * wave;
+  auto on_diagonal = [&](uint32_t n0) {
+    if constexpr (SPARSE) return false;
+    else return p.causal != 0 && n0 != OOB && (int)n0 + BN - 1 > wave_row0;
+  };
+  auto mask_tail = [&](floatx16& a0, floatx16& a1, int nvalid, uint32_t n0) {
+    int lim = nvalid;
+    if constexpr (!SPARSE) {
+      if (p.causal) lim = min(lim, my_row - (int)n0 + 1);
+    }
+    lim -= 4 * hh;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (8 * (r >> 2) + (r & 3) >= lim) a0[r] = -INFINITY;
+      if (8 * (r >> 2) + (r & 3) + 32 >= lim) a1[r] = -INFINITY;
+    }
+  };
+  auto across = [&](float x) {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+  };
+
+  vec8 f[8];
+  floatx16 sn0, sn1;
+  float mx = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+
+  if (have) {
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) dma_k1(0, n_cur, i);
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) dma_v1(0, n_cur, i);
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) dma_k1(1, n_nxt, i);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < 8; ++g) f[g] = read_k(sK, g & 1, g >> 1);
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
+      else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
+    }
+    if (v_cur < BN || on_diagonal(n_cur)) mask_tail(sn0, sn1, v_cur, n_cur);
+    float m2 = fmaxf(sn0[0], sn1[0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
+    mx = across(m2);
+  }
+
+  auto tile_step = [&](auto PAR) {
+    constexpr int par = decltype(PAR)::value;
+    const char* tV = sV + par * TILE64_BYTES;
+    const char* tKn = sK + (par ^ 1) * TILE64_BYTES;
+    floatx16 c0 = sn0, c1 = sn1;  // S(j)
+
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < 8; ++g) f[g] = read_k(tKn, g & 1, g >> 1);  // all of K(j+1), halves alternating
+
+    const float mx_s = mx * c;
+    if (__any(mx_s > m_run + RESCALE_SLACK)) {
+      const float m_new = fmaxf(m_run, mx_s);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+      m_run = m_new;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    uint32_t pk0[8], pk1[8];
+    float lsum = 0.f;
+    float tf[2][2], te[2][2];
+    auto expo_slot = [&](int n) {  // as in the head_dim-128 pipeline: a score pair takes three consecutive slots
+      if (n >= 2 && n < 18) {
+        const int j = n - 2;
+        lsum += te[j & 1][0] + te[j & 1][1];
+        (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
+      }
+      if (n >= 1 && n < 17) {
+        const int j = n - 1;
+        te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
+        te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
+      }
+      if (n < 16) {
+        const floatx16& cs = n < 8 ? c0 : c1;
+        tf[n & 1][0] = __builtin_fmaf(cs[2 * (n & 7)], c, -m_run);
+        tf[n & 1][1] = __builtin_fmaf(cs[2 * (n & 7) + 1], c, -m_run);
+      }
+    };
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+    // ---- stage A: S(j+1); slots 0..9 (P of keys 0..31 is complete when it ends) -----------------
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
+      else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
+      if (g < IPW) dma_k1(par, n_nx2, g);                      // K(j+2) takes the buffer K(j) has left
+      else if (g < 2 * IPW) dma_v1(par ^ 1, n_nxt, g - IPW);  // V(j+1) takes the buffer V(j-1) has left
+      f[g] = read_vt(tV, g >> 2, (g >> 1) & 1, g & 1);         // V(j) in the order stage B consumes it
+      if (g < 2) {
+        expo_slot(2 * g);
+        expo_slot(2 * g + 1);
+      } else {
+        expo_slot(g + 2);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (v_nxt < BN || on_diagonal(n_nxt)) mask_tail(sn0, sn1, v_nxt, n_nxt);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- stage B: O^T += V(j)^T P(j)^T; slots 10..17, then the row maximum of S(j+1) -------------
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int g = 2 * cc + db;
+        o[db] = T::mfma32(f[g], bfrag, o[db]);
+        expo_slot(10 + 2 * g);
+        expo_slot(11 + 2 * g);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    l_run += lsum;
+    float mxa = sn0[0], mxb = sn1[0];
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int g = 2 * cc + db;
+        o[db] = T::mfma32(f[4 + g], bfrag, o[db]);
+        mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g]), sn0[4 * g + 1]), sn0[4 * g + 2]), sn0[4 * g + 3]);
+        mxb = fmaxf(fmaxf(fmaxf(fmaxf(mxb, sn1[4 * g]), sn1[4 * g + 1]), sn1[4 * g + 2]), sn1[4 * g + 3]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    mx = across(fmaxf(mxa, mxb));
+
+    n_cur = n_nxt;
+    v_cur = v_nxt;
+    n_nxt = n_nx2;
+    v_nxt = v_nx2;
+    pull(n_nx2, v_nx2);
+    have = n_cur != OOB;
+  };
+
+  while (have) {
+    tile_step(std::integral_constant<int, 0>{});
+    if (!have) break;
+    tile_step(std::integral_constant<int, 1>{});
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the wavefront ends
+
+  float l_tot;
+  {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+    l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  }
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  if (row_ok) {
+    uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)my_row * p.os_s;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        u32x2 w;
+        w[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
+        w[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
+        *(u32x2*)(op + 32 * db + 8 * a + 4 * hh) = w;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      p.lse[((int64_t)batch * p.H + head) * p.Sq + my_row] = lse;
+    }
+  }
+}
+
 // Folds the split_s partial results of each split query tile into out and lse: the log-sum-exp
 // merge of torch's _SDPAMerger (used by src/para_attn/sparse_attn.py:174-189) over all pieces at
 // once.  One thread = 8 consecutive output elements of one query row; 16 rows per workgroup.
@@ -1444,6 +1774,11 @@ template <typename T, int D, bool SPARSE>
 static int launch_attn(const AttnParams& p, hipStream_t stream) {
   int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
   if (nblocks == 0) return PA_OK;
+  // only the head_dim-128 pipelined kernel folds into a running pair or splits keys; the others would
+  // store through the (absent) plain output
+  if ((p.acc_out != nullptr || p.split_s > 1) && !(D == 128 && p.pipe && !SPARSE))
+    PA_FAIL(PA_ERR_UNSUPPORTED, "accumulation / key split reached a kernel that has neither");
+  if (p.out == nullptr && p.acc_out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
   if (p.split_s > 1) nblocks = (int64_t)p.split_main + (int64_t)p.split_tiles * p.split_s;
   if (p.xcd_chunk > 0) nblocks = 8 * (int64_t)p.xcd_chunk;
   const void* fn;
@@ -1455,9 +1790,9 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     else if (p.pipe) { fn = (const void*)attn_fwd_d128_pipe_kernel<T, SPARSE, 4>; slot = 1; }
     else { fn = (const void*)attn_fwd_d128_kernel<T, SPARSE>; slot = 0; }
   } else {
-    fn = (const void*)attn_fwd_kernel<T, D, SPARSE>;
-    smem = Smem<D>::BYTES;
-    slot = 0;
+    if (p.pipe && p.bm == 256) { fn = (const void*)attn_fwd_d64_pipe_kernel<T, SPARSE, 8>; slot = 2; smem = 4 * TILE64_BYTES; }
+    else if (p.pipe) { fn = (const void*)attn_fwd_d64_pipe_kernel<T, SPARSE, 4>; slot = 1; smem = 4 * TILE64_BYTES; }
+    else { fn = (const void*)attn_fwd_kernel<T, D, SPARSE>; slot = 0; smem = Smem<D>::BYTES; }
   }
   // the attribute belongs to the function on one device: remembered per device and kernel variant
   static bool attr_done[PA_MAX_DEVICES][3] = {};  // benign race: the call is idempotent
@@ -1475,7 +1810,12 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     else
       hipLaunchKernelGGL((attn_fwd_d128_kernel<T, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
   } else {
-    hipLaunchKernelGGL((attn_fwd_kernel<T, D, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+    if (slot == 2)
+      hipLaunchKernelGGL((attn_fwd_d64_pipe_kernel<T, SPARSE, 8>), dim3((unsigned)nblocks), dim3(512), smem, stream, p);
+    else if (slot == 1)
+      hipLaunchKernelGGL((attn_fwd_d64_pipe_kernel<T, SPARSE, 4>), dim3((unsigned)nblocks), dim3(256), smem, stream, p);
+    else
+      hipLaunchKernelGGL((attn_fwd_kernel<T, D, SPARSE>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
   }
   PA_CHECK_LAUNCH("attention kernel");
   if constexpr (D == 128 && !SPARSE) {
@@ -1541,14 +1881,18 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
   p.bm = 128;
   p.split_s = 0;
   auto finish = [&] { p.n_qtiles = (p.Sq + p.bm - 1) / p.bm; };
-  if (D != 128) return finish();
+  if (D != 128 && D != 64) return finish();
   if (p.Skv <= 0 || (uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB ||
       (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB)
     return finish();
-  if (env_is("PARAATTN_NO_PIPE", "1")) return finish();  // test aid: the kernel without offset limits
+  if (env_is("PARAATTN_NO_PIPE", "1")) return finish();  // test aid: the kernels without offset limits
   p.pipe = 1;
   const char* force = getenv("PARAATTN_BM");  // tuning aid
   const int forced = force ? atoi(force) : 0;
+  if (D == 64) {  // no key split at head_dim 64; 128 rows unless asked otherwise
+    if (forced == 256 && (dense || q_block % 256 == 0)) p.bm = 256;
+    return finish();
+  }
   if (!dense) {  // block-sparse: workgroups differ in length, no split
     if (forced == 256 && q_block % 256 == 0) p.bm = 256;
     return finish();
@@ -1619,7 +1963,7 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   choose_kernel(p, D, 256, true, workspace ? workspace_bytes : 0, nullptr);
   if (accumulate) {
     if (p.causal) PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation is not causal");
-    if (!p.pipe)
+    if (!p.pipe || D != 128)  // only the head_dim-128 pipelined kernel has the folding epilogue
       PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation needs head_dim 128 and K/V below 4 GiB per head; run pa_attn_fwd_lse and pa_merge_lse");
     p.acc_out = acc_out; p.acc_lse = acc_lse; p.acc_first = acc_first != 0;
     p.lse = nullptr;

@@ -66,6 +66,14 @@ def test_argument_validation_without_device_work():
     bad = (ctypes.c_int64 * 3)(0, 4096, 100)
     assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 1, 1, 16, 16, 128, bad, st, st, st, 1.0, None, 0, None) == _lib.PA_ERR_UNSUPPORTED
     assert lib.pa_attn_fwd_lse(None, a, a, a, None, 0, 1, 1, 16, 16, 128, st, st, st, st, 1.0, None, 0, None) == _lib.PA_ERR_INVALID
+    # the fused ring step exists for head_dim 128 only, is not causal, and says so before any launch
+    # (a head_dim-64 call once slipped through to a kernel without that epilogue and wrote through a null output)
+    st64 = (ctypes.c_int64 * 3)(0, 2048, 64)
+    assert lib.pa_attn_fwd_accumulate(a, a, a, a, a, None, 0, 1, 1, 16, 16, 64, st64, st64, st64, None, 1.0, None, 1,
+                                      None, 0, None) == _lib.PA_ERR_UNSUPPORTED
+    assert b"head_dim 128" in lib.pa_last_error()
+    assert lib.pa_attn_fwd_accumulate(a, a, a, None, a, None, 0, 1, 1, 16, 16, 128, st, st, st, None, 1.0, None, 1,
+                                      None, 0, None) == _lib.PA_ERR_INVALID
     # empty problems succeed without touching the device
     assert lib.pa_attn_fwd_lse(a, a, a, a, None, 0, 0, 1, 16, 16, 128, st, st, st, st, 1.0, None, 0, None) == _lib.PA_OK
     assert lib.pa_merge_lse(a, 2, a, a, 0, a, a, 2, a, 0, 128, None) == _lib.PA_OK

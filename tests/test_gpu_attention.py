@@ -160,13 +160,14 @@ def test_key_mask_and_sparse_kv(cuda):
 
 @pytest.mark.parametrize("env", [{"PARAATTN_NO_PIPE": "1"}, {"PARAATTN_BM": "256"}])
 def test_alternative_kernels(cuda, env, monkeypatch):
-    """The head_dim-128 kernel without 32-bit offset limits (taken when K or V spans 4 GiB or more) and the
-    8-wavefront workgroup variant compute the same thing as the default kernel."""
+    """The kernels without 32-bit offset limits (taken when K or V spans 4 GiB or more) and the 8-wavefront
+    workgroup variants compute the same thing as the default kernels, at head_dim 128 and 64."""
     import os
 
-    cases = [(1, 2, 300, 434), (2, 1, 129, 1000), (1, 1, 64, 64), (1, 3, 1000, 77)]
-    for B, H, Sq, Skv in cases:
-        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=Sq + Skv)
+    cases = [(1, 2, 300, 434, 128), (2, 1, 129, 1000, 128), (1, 1, 64, 64, 128), (1, 3, 1000, 77, 128),
+             (1, 2, 300, 434, 64), (2, 1, 129, 1000, 64), (1, 3, 1000, 77, 64)]
+    for B, H, Sq, Skv, D in cases:
+        q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=Sq + Skv)
         ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
         for name, val in env.items():
             monkeypatch.setenv(name, val)
@@ -250,15 +251,16 @@ def test_causal_vs_f64(cuda, B, H, Sq, Skv, D):
 
 @pytest.mark.parametrize("env", [{"PARAATTN_NO_PIPE": "1"}, {"PARAATTN_BM": "256"}, {"PARAATTN_BM": "128"}])
 def test_causal_alternative_kernels(cuda, env, monkeypatch):
-    for B, H, Sq, Skv in [(1, 2, 700, 700), (1, 1, 300, 90), (1, 2, 90, 300), (2, 1, 513, 513)]:
-        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=Sq + Skv)
+    for B, H, Sq, Skv, D in [(1, 2, 700, 700, 128), (1, 1, 300, 90, 128), (1, 2, 90, 300, 128), (2, 1, 513, 513, 128),
+                             (1, 2, 700, 700, 64), (1, 1, 300, 90, 64), (2, 1, 513, 513, 64)]:
+        q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=Sq + Skv)
         ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, oattn.causal_keep(Sq, Skv))
         for name, val in env.items():
             monkeypatch.setenv(name, val)
         out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), is_causal=True)
         for name in env:
             monkeypatch.delenv(name)
-        _check(out, lse, ref_out, ref_lse, f"causal {env} {(B, H, Sq, Skv)}")
+        _check(out, lse, ref_out, ref_lse, f"causal {env} {(B, H, Sq, Skv, D)}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -63,10 +63,11 @@ def test_runs_word_boundaries(cuda):
         assert got == want, i
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("per_head", [False, True])
 @pytest.mark.parametrize("qb,kb", [(128, 128), (64, 32), (50, 70), (200, 24)])
-def test_small_vs_masked_dense(cuda, per_head, qb, kb):
-    B, H, nQ, nK, D = 2, 3, 5, 6, 128
+def test_small_vs_masked_dense(cuda, per_head, qb, kb, D):
+    B, H, nQ, nK = 2, 3, 5, 6
     Sq, Skv = nQ * qb, nK * kb
     q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=qb + kb)
     mask, _ = inputs.block_mask(H if per_head else 1, nQ, nK, seed=1, window=0, sinks=1, density=0.5)
