@@ -286,6 +286,38 @@ def test_causal_argument_rules(cuda):
         torch.ops.para_attn.attention_forward_sparse_kv(q, k, v, mask, is_causal=True)
 
 
+def test_random_configurations(cuda):
+    """Sixty seeded random draws over shape, head_dim, dtype, layout, scale, is_causal and per-batch key counts,
+    each against the fp64 oracle: the combinations no hand-written case lists."""
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        B, H = int(rng.integers(1, 3)), int(rng.integers(1, 5))
+        Sq, Skv = int(rng.integers(1, 700)), int(rng.integers(1, 700))
+        D = int(rng.choice([64, 128]))
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+        causal = bool(rng.random() < 0.3)
+        use_len = (not causal) and bool(rng.random() < 0.3)
+        bshd = bool(rng.random() < 0.4)
+        scale = None if rng.random() < 0.6 else float(rng.uniform(0.02, 0.3))
+        q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=1000 + case, dtype=dtype)
+        keep = None
+        mask = None
+        if causal:
+            keep = oattn.causal_keep(Sq, Skv)
+        elif use_len:
+            lens = rng.integers(1, Skv + 1, size=B)
+            kb = np.arange(Skv)[None, :] < lens[:, None]
+            keep = kb[:, None, None, :]
+            mask = torch.from_numpy(kb)[:, None, None, :].to(cuda)
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale, keep)
+        qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+        if bshd:  # [B,S,H,D] memory behind a [B,H,S,D] view
+            qd, kd, vd = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (qd, kd, vd))
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, mask, is_causal=causal, scale=scale)
+        what = f"case {case}: B{B} H{H} Sq{Sq} Skv{Skv} D{D} {dtype} causal={causal} len={use_len} bshd={bshd} scale={scale}"
+        _check(out, lse, ref_out, ref_lse, what)
+
+
 def test_key_rows_spread_over_4gib(cuda):
     """K and V whose rows lie 1 MiB apart span more than 4 GiB per head: beyond the 32-bit offsets of the
     pipelined kernel, so the launch must pick the kernel without that limit (a wrong pick reads zeros)."""
