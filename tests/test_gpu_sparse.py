@@ -133,3 +133,35 @@ def test_config5_shape_sampled(cuda):
             np.testing.assert_allclose(lse[:, h : h + 1, rows].cpu().numpy(), rl.numpy(), atol=1e-3)
             np.testing.assert_allclose(out[:, h : h + 1, rows].float().cpu().numpy(), ro.float().numpy(), atol=2e-2, rtol=2e-2)
     assert torch.isfinite(out.float()).all()
+
+
+def test_random_configurations(cuda):
+    """Forty seeded random draws over block sizes, block counts, dense margins, mask density (rows that keep
+    nothing included), per-head masks, head_dim and dtype, each against dense attention with -inf on the dropped tiles."""
+    rng = np.random.default_rng(77)
+    for case in range(40):
+        B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+        D = int(rng.choice([64, 128]))
+        dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
+        nQ, nK = int(rng.integers(1, 7)), int(rng.integers(1, 9))
+        qb, kb = int(rng.choice([8, 37, 64, 128, 130, 256])), int(rng.choice([5, 32, 64, 100, 128]))
+        q_lo, q_tail = (int(rng.integers(0, 90)), int(rng.integers(0, 90))) if rng.random() < 0.5 else (0, 0)
+        kv_lo, kv_tail = (int(rng.integers(0, 90)), int(rng.integers(0, 90))) if rng.random() < 0.5 else (0, 0)
+        Sq, Skv = q_lo + nQ * qb + q_tail, kv_lo + nK * kb + kv_tail
+        per_head = bool(rng.random() < 0.4)
+        dens = float(rng.choice([0.1, 0.3, 0.6, 1.0]))
+        bm = torch.from_numpy(rng.random((H if per_head else 1, nQ, nK)) < dens)
+        bm2 = bm if per_head else bm[0]
+        q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=500 + case, dtype=dtype)
+        q_range, kv_range = (q_lo, q_lo + nQ * qb), (kv_lo, kv_lo + nK * kb)
+        keep = osparse.expand_block_mask(bm2.numpy(), Sq, Skv, q_range, kv_range)
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, keep)
+        out, lse = torch.ops.para_attn.attention_forward_block_sparse(
+            q.to(cuda), k.to(cuda), v.to(cuda), bm2.to(cuda), q_range[0], q_range[1], kv_range[0], kv_range[1])
+        what = f"case {case}: B{B} H{H} D{D} {dtype} nQ{nQ}x{qb} nK{nK}x{kb} margins q({q_lo},{q_tail}) kv({kv_lo},{kv_tail}) per_head={per_head} density={dens}"
+        got_lse = lse.cpu().numpy().astype(np.float64)
+        both_inf = np.isneginf(got_lse) & np.isneginf(ref_lse)
+        assert (np.isneginf(got_lse) == np.isneginf(ref_lse)).all(), what
+        assert (np.abs(np.where(both_inf, 0.0, got_lse - np.where(both_inf, 0.0, ref_lse))) <= 1e-3).all(), what
+        err = np.abs(out.float().cpu().numpy().astype(np.float64) - ref_out)
+        assert (err <= 2e-2 + 2e-2 * np.abs(ref_out)).all(), what + f" max err {err.max():.4g}"
