@@ -102,7 +102,7 @@ def _dense_forward(query, key, value, scale, want_lse, kv_len=None, is_causal=Fa
         # scratch for the key-split tail of the launch (torch's caching allocator: no hipMalloc in
         # the steady state); its lifetime on the launch stream is the allocator's business
         ks, vs = _lib.strides3(k), _lib.strides3(v)
-        ws_bytes = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, ks, vs)
+        ws_bytes = 0 if is_causal else lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, ks, vs)  # causal launches never split
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
         rc = lib.pa_attn_fwd_lse_ws(
             _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
