@@ -2,12 +2,13 @@
 (src/para_attn/first_block_cache/utils.py:12-120, 193-295): the cache context,
 the gates of ``get_can_use_cache`` and ``are_two_tensors_similar``, whose
 seven-launch reduction is one kernel here, and the TaylorSeer variant of the
-cached residual (utils.py:297-312).  The diffusers adapters and the block
-orchestration are not part of this package.
+cached residual (utils.py:297-312), and ``CachedTransformerBlocks``, the module the
+reference's adapters swap in for a model's block list (utils.py:333-451).  The
+diffusers adapters themselves are not part of this package.
 """
 import contextlib
 import dataclasses
-from typing import Any, Dict, Optional, Union
+from typing import Any, Dict, List, Optional, Union
 
 import torch
 
@@ -27,6 +28,9 @@ class CacheContext:
     warmup_steps: int = 0
     enable_taylorseer: bool = False
     taylorseer_kwargs: Dict[str, Any] = dataclasses.field(default_factory=dict)
+    slg_layers: Optional[List[int]] = None
+    slg_start: float = 0.0
+    slg_end: float = 0.1
     taylorseer: Optional[TaylorSeer] = None
     alter_taylorseer: Optional[TaylorSeer] = None
     buffers: Dict[str, Any] = dataclasses.field(default_factory=dict)
@@ -77,6 +81,22 @@ class CacheContext:
                 self.executed_steps += 1
         if self.enable_taylorseer:
             self.get_taylorseer().mark_step_begin()
+
+    def is_slg_enabled(self):
+        return self.slg_layers is not None
+
+    def slg_should_skip_block(self, block_idx):
+        """utils.py:102-114: skip-layer guidance drops the listed blocks on the alternating pass, inside
+        the step window [slg_start, slg_end) of the schedule."""
+        if not self.enable_alter_cache or not self.is_alter_cache:
+            return False
+        if self.slg_layers is None:
+            return False
+        if self.slg_start <= 0.0 and self.slg_end >= 1.0:
+            return False
+        assert self.num_inference_steps >= 0, "num_inference_steps must be non-negative"
+        n = self.num_inference_steps
+        return block_idx in self.slg_layers and n * self.slg_start <= self.get_current_step() < n * self.slg_end
 
     def get_current_step(self):
         return self.executed_steps - 1
@@ -252,3 +272,102 @@ def set_encoder_hidden_states_residual(encoder_hidden_states_residual):
 @torch.compiler.disable
 def get_encoder_hidden_states_residual():
     return _ctx().get_buffer("encoder_hidden_states_residual")
+
+
+@torch.compiler.disable
+def mark_step_begin():
+    _ctx().mark_step_begin()
+
+
+@torch.compiler.disable
+def is_slg_enabled():
+    return _ctx().is_slg_enabled()
+
+
+@torch.compiler.disable
+def slg_should_skip_block(block_idx):
+    return _ctx().slg_should_skip_block(block_idx)
+
+
+def _residual(after, before):
+    """``after - before`` as one kernel, contiguous (utils.py:443-449)."""
+    return ops.fbcache_first_residual_diff(after, before, None)[0]
+
+
+class CachedTransformerBlocks(torch.nn.Module):
+    """The caller of the First Block Cache path (src/para_attn/first_block_cache/utils.py:333-451): run the
+    first block, decide from its residual whether the rest may be skipped, then either add the cached
+    residuals back or run the remaining blocks and cache theirs.  Constructor and return conventions are
+    the reference's; the residual, the reduction and the decision are one kernel (``first_block_step``),
+    the cache hit another, the residuals of the remaining blocks one each."""
+
+    def __init__(self, transformer_blocks, single_transformer_blocks=None, *, transformer=None,
+                 return_hidden_states_first=True, return_hidden_states_only=False):
+        super().__init__()
+        self.transformer = transformer
+        self.transformer_blocks = transformer_blocks
+        self.single_transformer_blocks = single_transformer_blocks
+        self.return_hidden_states_first = return_hidden_states_first
+        self.return_hidden_states_only = return_hidden_states_only
+
+    def _dual(self, block, hidden_states, encoder_hidden_states, *args, **kwargs):
+        """A block returns the hidden states alone, or both streams in the order the model uses."""
+        out = block(hidden_states, encoder_hidden_states, *args, **kwargs)
+        if isinstance(out, torch.Tensor):
+            return out, encoder_hidden_states
+        first, second = out
+        return (first, second) if self.return_hidden_states_first else (second, first)
+
+    def forward(self, hidden_states, encoder_hidden_states, *args, **kwargs):
+        original_hidden_states = hidden_states
+        hidden_states, encoder_hidden_states = self._dual(
+            self.transformer_blocks[0], hidden_states, encoder_hidden_states, *args, **kwargs)
+        parallelized = self.transformer is not None and getattr(self.transformer, "_is_parallelized", False)
+        first_residual, can_use_cache = first_block_step(hidden_states, original_hidden_states, parallelized)
+        del original_hidden_states
+
+        torch._dynamo.graph_break()
+        if can_use_cache:
+            del first_residual
+            hidden_states, encoder_hidden_states = apply_prev_hidden_states_residual(hidden_states, encoder_hidden_states)
+        else:
+            set_first_hidden_states_residual(first_residual)
+            del first_residual
+            hidden_states, encoder_hidden_states, res, enc_res = self.call_remaining_transformer_blocks(
+                hidden_states, encoder_hidden_states, *args, **kwargs)
+            set_hidden_states_residual(res)
+            set_encoder_hidden_states_residual(enc_res)
+        torch._dynamo.graph_break()
+
+        if self.return_hidden_states_only:
+            return hidden_states
+        if self.return_hidden_states_first:
+            return hidden_states, encoder_hidden_states
+        return encoder_hidden_states, hidden_states
+
+    def call_remaining_transformer_blocks(self, hidden_states, encoder_hidden_states, *args, **kwargs):
+        """utils.py:396-451: blocks 1.. of the dual-stream stack, then the single-stream stack on the
+        concatenated sequence; blocks named by skip-layer guidance are left out."""
+        original_hidden_states = hidden_states
+        original_encoder_hidden_states = encoder_hidden_states
+        slg = is_slg_enabled()
+        for i, block in enumerate(self.transformer_blocks[1:]):
+            if slg and slg_should_skip_block(i + 1):
+                continue
+            hidden_states, encoder_hidden_states = self._dual(block, hidden_states, encoder_hidden_states, *args, **kwargs)
+        if self.single_transformer_blocks is not None:
+            n_enc = encoder_hidden_states.shape[1]
+            hidden_states = torch.cat([encoder_hidden_states, hidden_states], dim=1)
+            for i, block in enumerate(self.single_transformer_blocks):
+                if slg and slg_should_skip_block(len(self.transformer_blocks) + i):
+                    continue
+                hidden_states = block(hidden_states, *args, **kwargs)
+            encoder_hidden_states, hidden_states = hidden_states.split([n_enc, hidden_states.shape[1] - n_enc], dim=1)
+
+        hidden_states = hidden_states.contiguous().reshape(original_hidden_states.shape)
+        res = _residual(hidden_states, original_hidden_states)
+        enc_res = None
+        if encoder_hidden_states is not None:
+            encoder_hidden_states = encoder_hidden_states.contiguous().reshape(original_encoder_hidden_states.shape)
+            enc_res = _residual(encoder_hidden_states, original_encoder_hidden_states)
+        return hidden_states, encoder_hidden_states, res, enc_res
