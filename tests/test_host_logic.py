@@ -206,3 +206,22 @@ def test_unified_attn_mode_on_cpu_passes_through():
 
     with pytest.raises(NotImplementedError):
         paraattention_amd.UnifiedAttnMode(FakeMesh())
+
+
+def test_skip_layer_guidance_window():
+    """utils.py:102-114: only on the alternating pass, only for listed blocks, only inside [start, end) of the schedule."""
+    from paraattention_amd import fbcache
+
+    ctx = fbcache.create_cache_context(slg_layers=[1, 3], enable_alter_cache=True, num_inference_steps=10, slg_start=0.1, slg_end=0.3)
+    assert ctx.is_slg_enabled() and not fbcache.create_cache_context().is_slg_enabled()
+    seen = []
+    for _ in range(10):  # plain / alter passes of steps 0..4
+        ctx.mark_step_begin()
+        seen.append((ctx.get_current_step(), ctx.is_alter_cache, ctx.slg_should_skip_block(1), ctx.slg_should_skip_block(2)))
+    assert seen == [(0, False, False, False), (0, True, False, False), (1, False, False, False), (1, True, True, False),
+                    (2, False, False, False), (2, True, True, False), (3, False, False, False), (3, True, False, False),
+                    (4, False, False, False), (4, True, False, False)]
+    whole = fbcache.create_cache_context(slg_layers=[1], enable_alter_cache=True, num_inference_steps=10, slg_start=0.0, slg_end=1.0)
+    whole.mark_step_begin()
+    whole.mark_step_begin()
+    assert whole.is_alter_cache and not whole.slg_should_skip_block(1)  # the degenerate window switches it off (utils.py:107-108)
