@@ -55,31 +55,107 @@ def _world_size(mesh):
     raise TypeError("mesh must be a ProcessGroup or DeviceMesh")
 
 
-class UnifiedAttnMode(TorchFunctionMode):
+def _sdpa(*args, **kwargs):
+    """The last stage on this GPU: the HIP kernel for the calls it takes, aten's SDPA for the rest."""
+    b = _bind(args, kwargs)
+    if kernel_takes(**b):
+        b.pop("enable_gqa", None)
+        return ops.attention_forward(**b)
+    return F.scaled_dot_product_attention(*args, **kwargs)
+
+
+def _one_rank(mesh, what):
+    if _world_size(mesh) > 1:
+        raise NotImplementedError(f"this build runs on one GPU: {what} over a mesh of more than one rank is not provided")
+
+
+def ulysses_attn_func(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None, mesh=None,
+                      attn_func=None):
+    """para_attn_interface.py:88-117 on one rank: the all-to-alls are identities, the attention remains."""
+    assert query.ndim == 4, "query must have 4 dimensions, got {}".format(query.ndim)
+    assert key.ndim == 4, "key must have 4 dimensions, got {}".format(key.ndim)
+    assert value.ndim == 4, "value must have 4 dimensions, got {}".format(value.ndim)
+    _one_rank(mesh, "ulysses attention")
+    fn = attn_func if attn_func is not None else _sdpa
+    return fn(query, key, value, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal, scale=scale)
+
+
+def ring_attn_func(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None, mesh=None):
+    """para_attn_interface.py:200-239 on one rank (world size <= 1 is plain attention there too, :213-222)."""
+    _one_rank(mesh, "ring attention")
+    return _sdpa(query, key, value, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal, scale=scale)
+
+
+def in_batch_attn_func(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
+    """para_attn_interface.py:242-276: the batch is folded into the sequence, so every image of the batch
+    attends the keys of all of them.  With [B,S,H,D] memory behind the [B,H,S,D] view (what diffusers hands
+    over) the fold is a view and the kernel reads it through its strides; otherwise torch copies once."""
+    assert query.ndim == 4, "query must have 4 dimensions, got {}".format(query.ndim)
+    assert key.ndim == 4, "key must have 4 dimensions, got {}".format(key.ndim)
+    assert value.ndim == 4, "value must have 4 dimensions, got {}".format(value.ndim)
+    assert attn_mask is None, "attn_mask is not supported in in_batch_attn_func"
+    assert not is_causal, "is_causal is not supported in in_batch_attn_func"
+    b, h, s_q, _ = query.shape
+    s_kv = value.shape[2]
+    query = query.permute(1, 0, 2, 3).reshape(1, h, b * s_q, -1)
+    key = key.permute(1, 0, 2, 3).reshape(1, h, b * s_kv, -1)
+    value = value.permute(1, 0, 2, 3).reshape(1, h, b * s_kv, -1)
+    out = _sdpa(query, key, value, attn_mask=None, dropout_p=dropout_p, is_causal=False, scale=scale)
+    return out.reshape(h, b, s_q, -1).permute(1, 0, 2, 3)
+
+
+class _SdpaMode(TorchFunctionMode):
+    """What the reference's modes share (src/para_attn/utils.py:19-32 and the class bodies): interception of
+    F.scaled_dot_product_attention, a class-wide ``disabled`` switch with ``disable()``."""
+
+    disabled = False
+
+    @torch.compiler.disable
+    def __init__(self, *, skip_small_kv=False):
+        super().__init__()
+        self._skip_small_kv = skip_small_kv
+
+    def _call(self, *args, **kwargs):
+        raise NotImplementedError
+
+    def __torch_function__(self, func, types, args=(), kwargs=None):
+        kwargs = {} if kwargs is None else kwargs
+        if type(self).disabled or func is not F.scaled_dot_product_attention:
+            return func(*args, **kwargs)
+        if self._skip_small_kv:
+            b = _bind(args, kwargs)
+            if b["query"].shape[-2] > b["key"].shape[-2]:  # more queries than keys: a cross-attention, left alone
+                return func(*args, **kwargs)
+        return self._call(*args, **kwargs)
+
+    @classmethod
+    @contextlib.contextmanager
+    def disable(cls):
+        old = cls._set_disabled(True)
+        try:
+            yield
+        finally:
+            cls._set_disabled(old)
+
+    @classmethod
+    @torch.compiler.disable
+    def _set_disabled(cls, value):
+        old = cls.disabled
+        cls.disabled = value
+        return old
+
+
+class UnifiedAttnMode(_SdpaMode):
     disabled = False
 
     @torch.compiler.disable
     def __init__(self, mesh=None, *, skip_small_kv=False, attn_func=None):
-        super().__init__()
-        if _world_size(mesh) > 1:
-            raise NotImplementedError("this build runs on one GPU: ulysses / ring meshes of more than one rank are not provided")
+        super().__init__(skip_small_kv=skip_small_kv)
+        _one_rank(mesh, "ulysses / ring attention")
         self._parallel_method = "ulysses"
-        self._skip_small_kv = skip_small_kv
         self._attn_func = attn_func
 
-    def __torch_function__(self, func, types, args=(), kwargs=None):
-        kwargs = {} if kwargs is None else kwargs
-        if UnifiedAttnMode.disabled:
-            return func(*args, **kwargs)
-        if func is F.scaled_dot_product_attention:
-            if self._skip_small_kv:
-                b = _bind(args, kwargs)
-                if b["query"].shape[-2] > b["key"].shape[-2]:
-                    return func(*args, **kwargs)
-            return self._call_unified_attn_func(*args, **kwargs)
-        return func(*args, **kwargs)
-
-    def _call_unified_attn_func(self, *args, **kwargs):
+    def _call(self, *args, **kwargs):
         func = F.scaled_dot_product_attention
         method = self._parallel_method
         if method in ("ulysses", "ring"):  # world size 1: both stages pass the call on
@@ -95,27 +171,48 @@ class UnifiedAttnMode(TorchFunctionMode):
             return ops.attention_forward(*args, **kwargs)
         if self._attn_func is not None:
             return self._attn_func(*args, **kwargs)
-        if kernel_takes(**_bind(args, kwargs)):
-            b = _bind(args, kwargs)
-            b.pop("enable_gqa", None)
-            return ops.attention_forward(**b)
-        return func(*args, **kwargs)
+        return _sdpa(*args, **kwargs)
 
-    @classmethod
-    @contextlib.contextmanager
-    def disable(cls):
-        old = cls._set_disabled(True)
-        try:
-            yield
-        finally:
-            cls._set_disabled(old)
 
-    @classmethod
+class RingAttnMode(_SdpaMode):
+    """para_attn_interface.py:303-350."""
+
+    disabled = False
+
     @torch.compiler.disable
-    def _set_disabled(cls, value):
-        old = cls.disabled
-        cls.disabled = value
-        return old
+    def __init__(self, mesh=None, *, skip_small_kv=False):
+        super().__init__(skip_small_kv=skip_small_kv)
+        _one_rank(mesh, "ring attention")
+
+    def _call(self, *args, **kwargs):
+        return ring_attn_func(*args, **kwargs)
+
+
+class UlyssesAttnMode(_SdpaMode):
+    """para_attn_interface.py:353-392."""
+
+    disabled = False
+
+    @torch.compiler.disable
+    def __init__(self, mesh=None, *, skip_small_kv=False):
+        super().__init__(skip_small_kv=skip_small_kv)
+        _one_rank(mesh, "ulysses attention")
+
+    def _call(self, *args, **kwargs):
+        return ulysses_attn_func(*args, **kwargs)
+
+
+class InBatchAttnMode(_SdpaMode):
+    """para_attn_interface.py:498-530."""
+
+    disabled = False
+
+    @torch.compiler.disable
+    def __init__(self):
+        super().__init__()
+
+    def _call(self, *args, **kwargs):
+        return in_batch_attn_func(*args, **kwargs)
 
 
 def sparse_kv_attn_func(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None,
@@ -126,7 +223,7 @@ def sparse_kv_attn_func(query, key, value, attn_mask=None, dropout_p=0.0, is_cau
                                            is_causal=is_causal, scale=scale)
 
 
-class SparseKVAttnMode(TorchFunctionMode):
+class SparseKVAttnMode(_SdpaMode):
     """src/para_attn/sparse_attn.py:607-640."""
 
     disabled = False
@@ -136,26 +233,5 @@ class SparseKVAttnMode(TorchFunctionMode):
         super().__init__()
         self._dispatch_to_custom_ops = dispatch_to_custom_ops
 
-    def __torch_function__(self, func, types, args=(), kwargs=None):
-        kwargs = {} if kwargs is None else kwargs
-        if SparseKVAttnMode.disabled:
-            return func(*args, **kwargs)
-        if func is F.scaled_dot_product_attention:
-            return sparse_kv_attn_func(*args, **kwargs, dispatch_to_custom_ops=self._dispatch_to_custom_ops)
-        return func(*args, **kwargs)
-
-    @classmethod
-    @contextlib.contextmanager
-    def disable(cls):
-        old = cls._set_disabled(True)
-        try:
-            yield
-        finally:
-            cls._set_disabled(old)
-
-    @classmethod
-    @torch.compiler.disable
-    def _set_disabled(cls, value):
-        old = cls.disabled
-        cls.disabled = value
-        return old
+    def _call(self, *args, **kwargs):
+        return sparse_kv_attn_func(*args, **kwargs, dispatch_to_custom_ops=self._dispatch_to_custom_ops)

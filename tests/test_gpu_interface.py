@@ -90,3 +90,35 @@ def test_compiled_ops_fullgraph(cuda):
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
     full, lse = torch.ops.para_attn.attention_forward_with_lse(q, k, v)
     assert (got[0].float() - full.float()).abs().max().item() <= 2e-2 and (got[1] - lse).abs().max().item() <= 1e-3
+
+
+def test_in_batch_ring_and_ulysses_on_one_rank(cuda):
+    """para_attn_interface.py:88-117, 200-276: on one rank ring and ulysses attention are plain attention, and
+    in-batch attention lets every batch element attend the keys of all of them."""
+    B, H, Sq, Skv, D = 3, 2, 70, 90, 128
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=8)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    direct = torch.ops.para_attn.attention_forward(qd, kd, vd)
+    assert torch.equal(paraattention_amd.ring_attn_func(qd, kd, vd), direct)
+    assert torch.equal(paraattention_amd.ulysses_attn_func(qd, kd, vd), direct)
+    with paraattention_amd.RingAttnMode():
+        assert torch.equal(F.scaled_dot_product_attention(qd, kd, vd), direct)
+    with paraattention_amd.UlyssesAttnMode(skip_small_kv=True):
+        assert torch.equal(F.scaled_dot_product_attention(qd, kd, vd), direct)
+    # in-batch: queries of every element against the concatenated keys of all elements
+    kf = k.permute(1, 0, 2, 3).reshape(1, H, B * Skv, D).float().numpy()
+    vf = v.permute(1, 0, 2, 3).reshape(1, H, B * Skv, D).float().numpy()
+    qf = q.permute(1, 0, 2, 3).reshape(1, H, B * Sq, D).float().numpy()
+    ref, _ = oattn.sdpa_lse_f64(qf, kf, vf)
+    ref = ref.reshape(H, B, Sq, D).transpose(1, 0, 2, 3)
+    out = paraattention_amd.in_batch_attn_func(qd, kd, vd)
+    assert out.shape == (B, H, Sq, D)
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref, atol=2e-2, rtol=2e-2)
+    with paraattention_amd.InBatchAttnMode():
+        out2 = F.scaled_dot_product_attention(qd, kd, vd)
+    assert torch.equal(out2, out)
+    # [B,S,H,D] memory: the fold is a view, no copy of q, k or v is made
+    qs, ks, vs = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (qd, kd, vd))
+    folded = qs.permute(1, 0, 2, 3).reshape(1, H, B * Sq, D)
+    assert folded.data_ptr() == qs.data_ptr()
+    assert torch.equal(paraattention_amd.in_batch_attn_func(qs, ks, vs), out)
