@@ -1730,8 +1730,11 @@ using namespace pa;
 static int check_common(const void* q, const void* k, const void* v, void* out, int dtype, int B,
                         int H, int Sq, int Skv, int D, const int64_t* qs, const int64_t* ks,
                         const int64_t* vs, const int64_t* os, float scale) {
-  if (!q || !k || !v || !out || !qs || !ks || !vs || !os) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
   if (B < 0 || H < 0 || Sq < 0 || Skv < 0) PA_FAIL(PA_ERR_INVALID, "negative size");
+  // an operand without elements may come as a null pointer (torch hands out none for empty tensors)
+  const bool any_row = B > 0 && H > 0 && Sq > 0;
+  if (!qs || !ks || !vs || !os || (any_row && (!q || !out)) || (any_row && Skv > 0 && (!k || !v)))
+    PA_FAIL(PA_ERR_INVALID, "null pointer argument");
   if (dtype != PA_DTYPE_BF16 && dtype != PA_DTYPE_F16)
     PA_FAIL(PA_ERR_UNSUPPORTED, "attention dtype must be bf16 or f16 (got code %d)", dtype);
   if (D != 128 && D != 64) PA_FAIL(PA_ERR_UNSUPPORTED, "head_dim %d not supported (64 or 128)", D);

@@ -158,6 +158,23 @@ def test_key_mask_and_sparse_kv(cuda):
         _check(out, lse, ref_out, ref_lse, "key mask")
 
 
+@pytest.mark.parametrize("D", [128, 64])
+def test_empty_inputs(cuda, D):
+    """No keys at all (Skv = 0, or a batch element whose mask keeps nothing): out = 0 and lse = -inf, what the
+    softmax over an empty set sums to; no queries: empty outputs; all without touching memory out of bounds."""
+    q, k, v = (t.to(cuda) for t in inputs.qkv(2, 2, 70, 50, D, seed=2))
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q, k[:, :, :0], v[:, :, :0])
+    assert out.shape == q.shape and (out == 0).all() and torch.isneginf(lse).all()
+    keep = torch.zeros(2, 1, 1, 50, dtype=torch.bool, device=cuda)
+    keep[0] = True
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q, k, v, keep)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q[:1].float().cpu().numpy(), k[:1].float().cpu().numpy(), v[:1].float().cpu().numpy())
+    _check(out[:1], lse[:1], ref_out, ref_lse, "kept batch element")
+    assert (out[1] == 0).all() and torch.isneginf(lse[1]).all()
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q[:, :, :0], k, v)
+    assert out.shape == (2, 2, 0, D) and lse.shape == (2, 2, 0)
+
+
 @pytest.mark.parametrize("env", [{"PARAATTN_NO_PIPE": "1"}, {"PARAATTN_BM": "256"}])
 def test_alternative_kernels(cuda, env, monkeypatch):
     """The kernels without 32-bit offset limits (taken when K or V spans 4 GiB or more) and the 8-wavefront
