@@ -7,9 +7,10 @@ resident in HBM (a call = the attention kernel plus the 8 us merge of its key-sp
 against) on a bounded sample of the same workload; ``extras`` holds the bandwidth-bound kernels
 (ring merge step, FBCache reduction) against the HBM peak and the block-sparse mode.
 
-``--only {attn,merge,fbcache,taylorseer,sparse,ring}`` runs a single kernel's loop (what the rocprofv3 summaries
-under profiles/ were taken with); the ring sweep launches the headline kernel at another shape, so it is
-kept out of the default run, whose per-kernel averages then describe one workload each.
+``--only {attn,merge,fbcache,taylorseer,sparse,ring,shapes}`` runs a single kernel's loop (what the rocprofv3
+summaries under profiles/ were taken with); the ring sweep and ``shapes`` (the dense op at the other model
+shapes) launch the headline kernel at other shapes, so they are kept out of the default run, whose per-kernel
+averages then describe one workload each.
 """
 import argparse
 import json
@@ -136,6 +137,39 @@ def bench_ring(dev, steps=5, warmup=2):
     }
 
 
+def bench_shapes(dev, steps=10, warmup=3):
+    """The dense op at the other model shapes: FLUX, Wan self- and cross-attention, the headline shape with
+    is_causal, and a head_dim 64 shape.  Cross-attention to 512 keys sits near the ridge, so it gets both bounds."""
+    import torch
+
+    op = torch.ops.para_attn.attention_forward_with_lse
+    rows = []
+    cases = [
+        ("FLUX joint attention", 1, 24, 4608, 4608, 128, False),
+        ("Wan self-attention", 1, 40, 32760, 32760, 128, False),
+        ("Wan cross-attention to 512 text keys", 1, 40, 32760, 512, 128, False),
+        ("headline shape, is_causal", 1, 3, 119056, 119056, 128, True),
+        ("head_dim 64 (CogVideoX-like)", 1, 48, 17776, 17776, 64, False),
+    ]
+    for name, B, H, Sq, Skv, D, causal in cases:
+        g = torch.Generator().manual_seed(3)
+        q = torch.randn(B, H, Sq, D, generator=g).bfloat16().to(dev)
+        k = torch.randn(B, H, Skv, D, generator=g).bfloat16().to(dev)
+        v = torch.randn(B, H, Skv, D, generator=g).bfloat16().to(dev)
+        ms, _ = _time_calls(lambda: op(q, k, v, is_causal=causal), steps, warmup)
+        flops = 4.0 * B * H * Sq * Skv * D * (0.5 if causal else 1.0)  # causal: the kept half (Sq == Skv)
+        nbytes = 2.0 * B * H * D * (2 * Sq + 2 * Skv) + 4.0 * B * H * Sq
+        tf = flops / (ms * 1e-3) / 1e12
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        rows.append({
+            "workload": f"{name}: q [{B},{H},{Sq},{D}] k,v [{B},{H},{Skv},{D}] bf16", "ms_per_call": round(ms, 4),
+            "flop_per_call": flops, "tflops": round(tf, 1), "frac_mfma": round(tf / PEAK_BF16_TFLOPS, 4),
+            "bytes_per_call": nbytes, "gbs": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+        })
+        del q, k, v
+    return rows
+
+
 def bench_sparse(dev, steps=10, warmup=5):
     import torch
 
@@ -214,7 +248,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only", choices=["attn", "merge", "fbcache", "taylorseer", "sparse", "ring", "copy"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "fbcache", "taylorseer", "sparse", "ring", "shapes", "copy"], default=None,
                     help="profiling aid: run just one kernel's timed loop and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -229,9 +263,9 @@ def main():
     _lib.load()  # no fallback: a missing library is an error
     dev = torch.device("cuda:0")
 
-    if args.only in ("merge", "fbcache", "taylorseer", "sparse", "ring", "copy"):
+    if args.only in ("merge", "fbcache", "taylorseer", "sparse", "ring", "shapes", "copy"):
         fn = {"merge": bench_merge, "fbcache": bench_fbcache, "taylorseer": bench_taylorseer, "sparse": bench_sparse,
-              "ring": bench_ring, "copy": bench_copy}[args.only]
+              "ring": bench_ring, "shapes": bench_shapes, "copy": bench_copy}[args.only]
         print(json.dumps({args.only: fn(dev, args.steps, args.warmup)}))
         return
 
