@@ -1851,18 +1851,23 @@ struct SplitPlan {
   int tiles, s;
   double rounds;
 };
-static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, bool allow) {
+static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bool allow) {
   if (slots <= 0) return {0, 1, 1.0};  // no device to ask: no estimate, no split
   SplitPlan best = {0, 1, (double)((n_tiles + slots - 1) / slots)};
   if (!allow || n_tiles % slots == 0) return best;
   SplitPlan found = best;
   double best_found = best.rounds;
+  // one round in microseconds (a key tile takes a workgroup about 1.75 us), to price the merge launch in
+  // rounds: about 8 us of launch gap plus its partials at 3 TB/s (measured: 17.7 us for 46 MB; at 4608 keys
+  // that is 0.13 of a round and the split loses, at 119k keys 0.03 and it wins)
+  const double round_us = ((double)kv_tiles + 4.0) * 1.75;
   for (int extra = 0; extra < 2; ++extra) {
     const int64_t T = n_tiles % slots + (int64_t)extra * slots;
     if (T > n_tiles || T * 8 > 0x7fffffffLL) break;
     for (int s = 2; s <= 8 && kv_tiles / s >= 16; ++s) {
       const double share = ((double)kv_tiles / s + 4.0) / ((double)kv_tiles + 4.0);
-      const double r = (double)((n_tiles - T) / slots) + (double)((T * s + slots - 1) / slots) * share + 0.02;
+      const double merge_us = 8.0 + (double)T * s * bm * 129.0 * 4.0 / 3.0e6;
+      const double r = (double)((n_tiles - T) / slots) + (double)((T * s + slots - 1) / slots) * share + merge_us / round_us;
       if (r < best.rounds * 0.97 && r < best_found) { best_found = r; found = {(int)T, s, r}; }
     }
   }
@@ -1914,10 +1919,10 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
   const int kv_tiles = (p.Skv + BN - 1) / BN;
   const int64_t bh = (int64_t)p.B * p.H;
   const int64_t n128 = bh * ((p.Sq + 127) / 128), n256 = bh * ((p.Sq + 255) / 256);
-  SplitPlan p128 = plan_split(n128, 2 * cus, kv_tiles, allow), p256 = plan_split(n256, cus, kv_tiles, allow);
+  SplitPlan p128 = plan_split(n128, 2 * cus, kv_tiles, 128, allow), p256 = plan_split(n256, cus, kv_tiles, 256, allow);
   if (!ws_needed) {  // the plan must fit what was lent
-    if (split_ws_bytes(p128, 128) > ws_bytes) p128 = plan_split(n128, 2 * cus, kv_tiles, false);
-    if (split_ws_bytes(p256, 256) > ws_bytes) p256 = plan_split(n256, cus, kv_tiles, false);
+    if (split_ws_bytes(p128, 128) > ws_bytes) p128 = plan_split(n128, 2 * cus, kv_tiles, 128, false);
+    if (split_ws_bytes(p256, 256) > ws_bytes) p256 = plan_split(n256, cus, kv_tiles, 256, false);
   }
   // an unsplit last round of 128-row workgroups that leaves every CU at most one of them runs
   // about 1.5 times faster per workgroup
