@@ -889,7 +889,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     const uint16_t* qp = qbase + (int64_t)r * p.qs_s + 8 * hh;
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): keep Q out of the loop's wait accounting
+    // no wait here: the loads overlap the first tile copies, whose wait in front of the first barrier covers them
   }
 
   // ---- global -> LDS copies: raw buffer loads with the LDS bit ---------------------------------
@@ -1318,7 +1318,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
     const uint16_t* qp = qbase + (int64_t)r * p.qs_s + 8 * hh;
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): keep Q out of the loop's wait accounting
+    // no wait here: the loads overlap the first tile copies, whose wait in front of the first barrier covers them
   }
 
   // global -> LDS copies as in the head_dim-128 pipeline: wave w, step i covers tile rows
