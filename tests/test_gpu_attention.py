@@ -133,6 +133,35 @@ def test_hunyuan_shape_sampled_rows(cuda):
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
 
 
+def test_hunyuan_shape_every_row_by_closed_forms(cuda):
+    """Properties that hold whatever the size, checked on every query row of the 119k-token shape (the sampled-row
+    test above leaves most rows to chance): with zero keys every score is 0, so LSE = ln(Skv) and out = the mean
+    of V over the keys; with V constant along the keys, out is that constant whatever the scores; and out is
+    linear in V at fixed q, k while LSE does not depend on V."""
+    B, H, S, D = 1, 3, 119056, 128
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=5, rms_norm_qk=True)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    op = torch.ops.para_attn.attention_forward_with_lse
+    # zero keys
+    out, lse = op(qd, torch.zeros_like(kd), vd)
+    assert (lse - np.log(S)).abs().max().item() <= 1e-3
+    mean_v = vd.float().mean(dim=2, keepdim=True)  # [B,H,1,D]
+    assert (out.float() - mean_v).abs().max().item() <= 2e-2
+    # V constant along the keys: row d of every key holds c[d]
+    c = torch.linspace(-2.0, 2.0, D).bfloat16().to(cuda)
+    out_c, lse_c = op(qd, kd, c.expand(B, H, S, D).contiguous())
+    assert (out_c.float() - c.float()).abs().max().item() <= 2e-2
+    # linearity in V; LSE independent of V
+    out1, lse1 = op(qd, kd, vd)
+    v2 = torch.roll(vd, 7, dims=2)
+    out2, lse2 = op(qd, kd, v2)
+    out3, lse3 = op(qd, kd, (0.5 * vd.float() - 0.25 * v2.float()).bfloat16())
+    assert torch.equal(lse1, lse2) and torch.equal(lse1, lse3) and torch.equal(lse1, lse_c)
+    # three bf16 roundings of outputs that are O(0.01) here; the bound is the parity tolerance itself
+    err = (out3.float() - (0.5 * out1.float() - 0.25 * out2.float())).abs()
+    assert (err <= 2e-2 + 2e-2 * out3.float().abs()).all(), err.max().item()
+
+
 def test_wan_cross_attention_shape(cuda):
     # the Wan 2.1 shape cross-attention: 32760 queries x 512 text keys (reduced heads for the CPU check)
     q, k, v = inputs.qkv(1, 4, 32760, 512, 128, seed=2)

@@ -145,3 +145,23 @@ def test_ring_sweep_full_shape_sampled(cuda):
         ro, rl = oattn.sdpa_lse_torch_cpu(q[:, h : h + 1, rows], kf, vf)
         np.testing.assert_allclose(lse[:, h : h + 1, rows.to(cuda)].cpu().numpy(), rl.numpy(), atol=1e-3)
         np.testing.assert_allclose(out[:, h : h + 1, rows.to(cuda)].float().cpu().numpy(), ro.float().numpy(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_ring_sweep_full_shape_every_row_by_closed_forms(cuda, fused):
+    """Every row of the ring-sweep shape, by properties that need no oracle run: with zero keys in all 8 blocks
+    LSE = ln(8 * 14882) and out = the mean of V over all blocks' keys; with V constant within a block the sweep
+    gives the mean of the blocks' constants."""
+    B, H, Sq, D, nblk = 1, 24, 14882, 128, 8
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(B, H, Sq, D, generator=g).bfloat16().to(cuda)
+    vb = [torch.randn(B, H, Sq, D, generator=g).bfloat16().to(cuda) for _ in range(nblk)]
+    zero = [torch.zeros(B, H, Sq, D, dtype=torch.bfloat16, device=cuda) for _ in range(nblk)]
+    out, lse = paraattention_amd.ring_sweep(q, zero, vb, fused=fused)
+    assert (lse - np.log(nblk * Sq)).abs().max().item() <= 1e-3
+    mean_v = torch.stack([t.float().mean(dim=2) for t in vb]).mean(dim=0)[:, :, None]  # equal block sizes
+    assert (out.float() - mean_v).abs().max().item() <= 2e-2
+    # V constant within a block, a different constant per block, zero keys: out = the mean of the constants
+    consts = [torch.full((B, H, Sq, D), float(i - 3), dtype=torch.bfloat16, device=cuda) for i in range(nblk)]
+    out_c, _ = paraattention_amd.ring_sweep(q, zero, consts, fused=fused)
+    assert (out_c.float() - (sum(range(nblk)) / nblk - 3.0)).abs().max().item() <= 2e-2

@@ -135,6 +135,29 @@ def test_config5_shape_sampled(cuda):
     assert torch.isfinite(out.float()).all()
 
 
+def test_config5_shape_every_row_by_closed_forms(cuda):
+    """Every row of the benchmark shape, by properties that need no oracle run: with zero keys all kept scores
+    are 0, so LSE = ln(number of kept keys) of the row's (head, query block) and out = the mean of V over the kept
+    keys; with V constant along the keys out is that constant."""
+    B, H, S, D, nb = 1, 24, 32768, 128, 256
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=3)
+    mask, _ = inputs.block_mask(H, nb, nb, seed=0)
+    qd, vd, md = q.to(cuda), v.to(cuda), mask.to(cuda)
+    op = torch.ops.para_attn.attention_forward_block_sparse
+    out, lse = op(qd, torch.zeros_like(qd), vd, md)
+    kept = mask.sum(dim=2).to(torch.float64) * (S // nb)                      # [H, nb] kept keys per query block
+    want_lse = torch.log(kept).repeat_interleave(S // nb, dim=1)[None]          # [1, H, S]
+    assert (lse.cpu().double() - want_lse).abs().max().item() <= 1e-3
+    # mean of V over the kept key blocks: block means [H, nb, D], averaged with the mask row as weights
+    blk_mean = vd.float().reshape(B, H, nb, S // nb, D).mean(dim=3)[0]          # [H, nb, D]
+    want_out = torch.einsum("hij,hjd->hid", md.float(), blk_mean) / md.float().sum(dim=2, keepdim=True)
+    want_out = want_out.repeat_interleave(S // nb, dim=1)[None]                 # [1, H, S, D]
+    assert (out.float() - want_out).abs().max().item() <= 2e-2
+    c = torch.linspace(-2.0, 2.0, D).bfloat16().to(cuda)
+    out_c, _ = op(qd, k.to(cuda), c.expand(B, H, S, D).contiguous(), md)
+    assert (out_c.float() - c.float()).abs().max().item() <= 2e-2
+
+
 def test_random_configurations(cuda):
     """Forty seeded random draws over block sizes, block counts, dense margins, mask density (rows that keep
     nothing included), per-head masks, head_dim and dtype, each against dense attention with -inf on the dropped tiles."""
