@@ -8,7 +8,8 @@ diffusers adapters themselves are not part of this package.
 """
 import contextlib
 import dataclasses
-from typing import Any, Dict, List, Optional, Union
+from collections import defaultdict
+from typing import Any, DefaultDict, Dict, List, Optional, Union
 
 import torch
 
@@ -34,6 +35,7 @@ class CacheContext:
     taylorseer: Optional[TaylorSeer] = None
     alter_taylorseer: Optional[TaylorSeer] = None
     buffers: Dict[str, Any] = dataclasses.field(default_factory=dict)
+    incremental_name_counters: DefaultDict[str, int] = dataclasses.field(default_factory=lambda: defaultdict(int))
     executed_steps: int = 0
     is_alter_cache: bool = True
 
@@ -42,6 +44,16 @@ class CacheContext:
             self.taylorseer = TaylorSeer(**self.taylorseer_kwargs)
             if self.enable_alter_cache:
                 self.alter_taylorseer = TaylorSeer(**self.taylorseer_kwargs)
+
+    def get_incremental_name(self, name=None):
+        """utils.py:45-50: "<name>_<count>", counting per name from 0."""
+        name = "default" if name is None else name
+        idx = self.incremental_name_counters[name]
+        self.incremental_name_counters[name] += 1
+        return f"{name}_{idx}"
+
+    def reset_incremental_names(self):
+        self.incremental_name_counters.clear()
 
     def get_taylorseer(self):
         if self.enable_alter_cache and self.is_alter_cache:
@@ -136,6 +148,30 @@ def _ctx():
     ctx = get_current_cache_context()
     assert ctx is not None, "cache_context must be set before"
     return ctx
+
+
+def get_residual_diff_threshold():
+    return _ctx().get_residual_diff_threshold()
+
+
+def get_buffer(name):
+    return _ctx().get_buffer(name)
+
+
+def set_buffer(name, buffer):
+    _ctx().set_buffer(name, buffer)
+
+
+def remove_buffer(name):
+    _ctx().remove_buffer(name)
+
+
+def is_in_warmup():
+    return _ctx().is_in_warmup()
+
+
+def get_downsample_factor():
+    return _ctx().downsample_factor
 
 
 def residual_diff(t1, t2):

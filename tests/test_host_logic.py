@@ -225,3 +225,34 @@ def test_skip_layer_guidance_window():
     whole.mark_step_begin()
     whole.mark_step_begin()
     assert whole.is_alter_cache and not whole.slg_should_skip_block(1)  # the degenerate window switches it off (utils.py:107-108)
+
+
+def test_cache_context_module_level_accessors():
+    """The module-level accessors of the reference (first_block_cache/utils.py:124-190, 263-267) read the current
+    context, respect the alternating cache's "_alter" buffer names and refuse to run without a context."""
+    with pytest.raises(AssertionError):
+        fbcache.get_buffer("x")
+    ctx = fbcache.create_cache_context(residual_diff_threshold=torch.tensor(0.12), alter_residual_diff_threshold=0.2,
+                                       enable_alter_cache=True, warmup_steps=2, downsample_factor=4)
+    with fbcache.cache_context(ctx):
+        assert fbcache.get_downsample_factor() == 4
+        # is_alter_cache starts True (utils.py:37): the alternating threshold and the "_alter" names apply
+        assert fbcache.get_residual_diff_threshold() == 0.2
+        fbcache.set_buffer("h", 1)
+        assert ctx.buffers == {"h_alter": 1} and fbcache.get_buffer("h") == 1
+        fbcache.mark_step_begin()  # flips to the main pass and counts a step
+        assert fbcache.get_residual_diff_threshold() == pytest.approx(0.12) and isinstance(fbcache.get_residual_diff_threshold(), float)
+        assert fbcache.get_buffer("h") is None
+        fbcache.set_buffer("h", 2)
+        fbcache.remove_buffer("h")
+        fbcache.remove_buffer("h")  # absent: no error (utils.py:74-78)
+        assert ctx.buffers == {"h_alter": 1}
+        assert fbcache.is_in_warmup()          # step 0 of 2 warm-up steps
+        for _ in range(4):
+            fbcache.mark_step_begin()          # two more counted steps
+        assert ctx.get_current_step() == 2 and not fbcache.is_in_warmup()
+    assert fbcache.get_current_cache_context() is None
+    # incremental names count per name from 0 (utils.py:45-53)
+    assert [ctx.get_incremental_name(), ctx.get_incremental_name(), ctx.get_incremental_name("a")] == ["default_0", "default_1", "a_0"]
+    ctx.reset_incremental_names()
+    assert ctx.get_incremental_name() == "default_0"
