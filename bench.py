@@ -292,7 +292,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "pa::attn_fwd_d128_pipe_kernel<pa::BF16, false, 8>",
+            "kernel": "pa::attn_fwd_d128_pipe_kernel<pa::BF16, false, 8, true>",
             "achieved": round(kern_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",

@@ -80,6 +80,14 @@ PA_API int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* ou
  * head_dim-128 kernel may compute the query tiles of the last, partly filled
  * round of workgroups in several key shares and fold them with the same
  * log-sum-exp merge as pa_merge_lse, which removes the idle tail of the launch.
+ * On launches of 2e12 flop and more the first 8 KB of the workspace hold a bound
+ * of the scores, computed on the device from the largest row norms of q and k
+ * (two small launches that read q and k once): where no score can leave
+ * [-60, 60] in the log2 domain (models that normalise q and k sit near 16) the
+ * kernel variant without a running maximum runs, about 4 % faster; otherwise,
+ * and always without a workspace, the variant with it.  Both are launched, and
+ * the one the device-side flag does not select returns at once, so nothing is
+ * read back by the host.
  * A null or short workspace is not an error: the call then runs as
  * pa_attn_fwd_lse does.  Results are the same to rounding.  Calls that share a
  * workspace must not overlap.
@@ -118,7 +126,7 @@ PA_API int pa_attn_fwd_accumulate(const void* q, const void* k, const void* v, f
 
 /*
  * Bytes of workspace pa_attn_fwd_lse_ws and pa_attn_fwd_accumulate can use for this problem on the current
- * device (0: it would not split).  Depends on the device's CU count.
+ * device (0: neither a key split nor a score bound would be used).  Depends on the device's CU count.
  */
 PA_API size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
                                    const int64_t k_strides[3], const int64_t v_strides[3]);

@@ -71,6 +71,9 @@ struct AttnParams {
   // consecutive shares of the key tiles, which leave normalised fp32 partial outputs and their
   // LSE in the workspace (piece-major) for attn_split_merge_kernel.  split_s <= 1: no split.
   int xcd_chunk;  // block-sparse pipelined kernel: ceil(workgroups / 8), 0 = plain order
+  // 256-row dense kernel: *bound_flag != 0 says that no score can leave [-60, 60] in the log2 domain (see
+  // score_bound_*_kernel), so the running maximum is not needed; null = not known, keep the maximum
+  const int* bound_flag;
   int split_main, split_tiles, split_s;
   float* ws_out;  // [split_s * split_tiles][bm][128]
   float* ws_lse;  // [split_s * split_tiles][bm]
@@ -830,11 +833,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 // workgroups in several key shares (AttnParams::split_*), fold the result into a running
 // (out, lse) pair (acc_*), or apply torch's causal mask (causal).
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool SPARSE, int NW>
+template <typename T, bool SPARSE, int NW, bool BOUNDED = false>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
   constexpr int DC = 8, DB = 4;
   constexpr int IPW = 16 / NW;  // copy instructions per wavefront and K (V) tile
+  // With a score bound on record the launch comes twice, once per variant, and the one the flag (computed on
+  // the device just before) does not select leaves at once.  BOUNDED: exp2(score) cannot overflow or vanish, so
+  // the reference point of the softmax stays 0 and row maxima, rescale checks and rescales are compiled out.
+  if constexpr (!SPARSE && NW == 8) {
+    if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
+  }
   constexpr int RS = 4 * NW;    // tile rows between two of them
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                    // [2][64][256 B]
@@ -966,7 +975,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   for (int i = 0; i < DB; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = BOUNDED ? 0.f : -INFINITY, l_run = 0.f;
   const float c = p.scale_log2;
 
   // window of tiles j (being consumed), j+1 and j+2: (first key or OOB, valid keys)
@@ -1042,10 +1051,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
     if (v_cur < BN || on_diagonal(n_cur)) mask_tail(sn0, sn1, v_cur, n_cur);
-    float m2 = fmaxf(sn0[0], sn1[0]);
+    if constexpr (!BOUNDED) {
+      float m2 = fmaxf(sn0[0], sn1[0]);
 #pragma unroll
-    for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
-    mx = across(m2);
+      for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
+      mx = across(m2);
+    }
   }
 
   // One iteration; PAR = buffer of tile j (K(j+1) sits in the other K buffer).
@@ -1063,16 +1074,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
 
-    const float mx_s = mx * c;
-    if (__any(mx_s > m_run + RESCALE_SLACK)) {
-      const float m_new = fmaxf(m_run, mx_s);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-      l_run *= alpha;
+    if constexpr (!BOUNDED) {
+      const float mx_s = mx * c;
+      if (__any(mx_s > m_run + RESCALE_SLACK)) {
+        const float m_new = fmaxf(m_run, mx_s);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        l_run *= alpha;
 #pragma unroll
-      for (int i = 0; i < DB; ++i)
+        for (int i = 0; i < DB; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
-      m_run = m_new;
+          for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+        m_run = m_new;
+      }
     }
     // Two 128-row workgroups share a CU unsynchronised: the wavefront that is in its second GEMM, where the
     // exponentials sit, gets the issue priority over the one that is in its first (+1.2 % measured; with one
@@ -1146,9 +1159,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         o[db] = T::mfma32(f[g], bfrag, o[db]);
         f[g] = read_vt(tV, 1, cc, db);  // keys 32..63
         if (g < 6) expo_slot(12 + g);
-        if (g < 4) {
-        } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
-        else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
+        if constexpr (!BOUNDED) {
+          if (g < 4) {
+          } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
+          else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -1160,12 +1175,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       for (int db = 0; db < DB; ++db) {
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
-        if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
+        if constexpr (!BOUNDED) {
+          if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
     l_run += lsum;
-    mx = across(fmaxf(mxa, mxb));
+    if constexpr (!BOUNDED) mx = across(fmaxf(mxa, mxb));
 
     // slide the tile window
     n_cur = n_nxt;
@@ -1736,6 +1753,82 @@ __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Score bound for the dense head_dim-128 kernel.  |q.k| <= |q| |k|, so with Mq = the largest row
+// norm of Q and Mk that of K no score leaves [-Mq Mk scale, Mq Mk scale]; in the log2 domain of the
+// kernel that is +-bound.  If bound <= `limit` (60 for bf16 P, whose exponent range is fp32's; 14
+// for fp16 P) then exp2(score) can neither overflow nor vanish, sums of up to 2^31 of them stay far
+// inside fp32, and the softmax needs no running maximum: a common factor 2^-m cancels in O / l and
+// in m + log2(l) whatever m is, so m = 0 gives the same results.  Models that normalise q and k
+// (RMS norm per head) sit near bound = 16.  Two launches: per-block maxima of the squared row
+// norms (blocks [0, G) over Q, [G, 2G) over K, 16 lanes per 256-byte row), then one block that
+// folds them and writes the flag.  An infinite element makes the bound infinite (flag 0); a NaN element
+// is not seen by the maxima, and its scores are NaN in either variant of the kernel.
+// ---------------------------------------------------------------------------------------------
+constexpr int BOUND_G = 1024;                                   // blocks per tensor
+constexpr size_t BOUND_WS_BYTES = (2 * BOUND_G + 64) * 4;       // partial maxima + the flag word (+ padding)
+
+template <typename T>
+__global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnParams p, float* part) {
+  const bool is_k = blockIdx.x >= BOUND_G;
+  const int blk = is_k ? blockIdx.x - BOUND_G : blockIdx.x;
+  const uint16_t* base = (const uint16_t*)(is_k ? p.k : p.q);
+  const int64_t sb = is_k ? p.ks_b : p.qs_b, sh = is_k ? p.ks_h : p.qs_h, ss = is_k ? p.ks_s : p.qs_s;
+  const int S = is_k ? p.Skv : p.Sq;
+  const int64_t rows = (int64_t)p.B * p.H * S;
+  const int sub = threadIdx.x & 15;
+  float best = 0.f;
+  for (int64_t r = (int64_t)blk * 16 + (threadIdx.x >> 4); r < rows; r += (int64_t)BOUND_G * 16) {
+    const int s_ = (int)(r % S);
+    const int64_t bh = r / S;
+    const uint16_t* rp = base + (bh / p.H) * sb + (bh % p.H) * sh + (int64_t)s_ * ss + 8 * sub;
+    const u32x4 w = *(const u32x4*)rp;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a = T::lo(w[i]), b = T::hi(w[i]);
+      acc = __builtin_fmaf(a, a, acc);
+      acc = __builtin_fmaf(b, b, acc);
+    }
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) acc += __shfl_xor(acc, d, 16);
+    best = fmaxf(best, acc);
+  }
+  __shared__ float sm[256];
+  sm[threadIdx.x] = best;
+  __syncthreads();
+  for (int d = 128; d > 0; d >>= 1) {
+    if ((int)threadIdx.x < d) {
+      sm[threadIdx.x] = fmaxf(sm[threadIdx.x], sm[threadIdx.x + d]);
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) part[blockIdx.x] = sm[0];
+}
+
+__global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part, float scale_log2, float limit, int* flag) {
+  __shared__ float sq[256], sk[256];
+  float mq = 0.f, mk = 0.f;
+  for (int i = threadIdx.x; i < BOUND_G; i += 256) {
+    mq = fmaxf(mq, part[i]);
+    mk = fmaxf(mk, part[BOUND_G + i]);
+  }
+  sq[threadIdx.x] = mq;
+  sk[threadIdx.x] = mk;
+  __syncthreads();
+  for (int d = 128; d > 0; d >>= 1) {
+    if ((int)threadIdx.x < d) {
+      sq[threadIdx.x] = fmaxf(sq[threadIdx.x], sq[threadIdx.x + d]);
+      sk[threadIdx.x] = fmaxf(sk[threadIdx.x], sk[threadIdx.x + d]);
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const float bound = sqrtf(sq[0]) * sqrtf(sk[0]) * scale_log2;
+    *flag = bound <= limit ? 1 : 0;
+  }
+}
+
 }  // namespace pa
 
 using namespace pa;
@@ -1784,6 +1877,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.causal = 0;
   p.acc_out = nullptr; p.acc_lse = nullptr; p.acc_first = 0;
   p.split_main = 0; p.split_tiles = 0; p.split_s = 0; p.ws_out = nullptr; p.ws_lse = nullptr;
+  p.bound_flag = nullptr;
 }
 
 template <typename T, int D, bool SPARSE>
@@ -1811,12 +1905,26 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     else { fn = (const void*)attn_fwd_kernel<T, D, SPARSE>; slot = 0; smem = Smem<D>::BYTES; }
   }
   // the attribute belongs to the function on one device: remembered per device and kernel variant
-  static bool attr_done[PA_MAX_DEVICES][3] = {};  // benign race: the call is idempotent
+  if (p.bound_flag != nullptr && !(D == 128 && slot == 2 && !SPARSE))
+    PA_FAIL(PA_ERR_UNSUPPORTED, "score bound reached a kernel that does not read it");
+  static bool attr_done[PA_MAX_DEVICES][4] = {};  // benign race: the call is idempotent
   const int dev = current_device();
   if (dev < 0 || !attr_done[dev][slot]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     if (dev >= 0) attr_done[dev][slot] = true;
+  }
+  if constexpr (D == 128 && !SPARSE) {
+    if (p.bound_flag != nullptr) {  // the variant without a running maximum first; one of the two returns at once
+      const void* fb = (const void*)attn_fwd_d128_pipe_kernel<T, false, 8, true>;
+      if (dev < 0 || !attr_done[dev][3]) {
+        hipError_t e = hipFuncSetAttribute(fb, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        if (dev >= 0) attr_done[dev][3] = true;
+      }
+      hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, false, 8, true>), dim3((unsigned)nblocks), dim3(512), smem, stream, p);
+      PA_CHECK_LAUNCH("attention kernel (bounded scores)");
+    }
   }
   if constexpr (D == 128) {
     if (slot == 2)
@@ -1960,6 +2068,16 @@ static int dispatch_attn(const AttnParams& p, int dtype, int D, hipStream_t stre
   return launch_attn<F16, 64, SPARSE>(p, stream);
 }
 
+// Whether a dense launch of this size is worth the two small launches that bound its scores (they read Q and K
+// once: about 45 us at the 119k-token shape, against 4 % of the attention kernel).  PARAATTN_BOUND=1 asks for the
+// bound at any size, =0 never (tuning and test aid).
+static bool bound_wanted(int B, int H, int Sq, int Skv, int D) {
+  if (D != 128 || B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0) return false;
+  if (env_is("PARAATTN_BOUND", "0")) return false;
+  if (env_is("PARAATTN_BOUND", "1")) return true;
+  return 4.0 * B * H * (double)Sq * (double)Skv * D >= 2.0e12;
+}
+
 static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out, float* lse,
                           int dtype, int B, int H, int Sq, int Skv, int D,
                           const int64_t q_strides[3], const int64_t k_strides[3],
@@ -1981,7 +2099,25 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
   p.kv_len = kv_len;
   p.causal = is_causal != 0;
-  choose_kernel(p, D, 256, true, workspace ? workspace_bytes : 0, nullptr);
+  // a workspace that has room for them beside the key split's partials starts with BOUND_WS_BYTES for the score bound
+  const size_t ws_avail = workspace ? workspace_bytes : 0;
+  char* ws_base = (char*)workspace;
+  choose_kernel(p, D, 256, true, ws_avail, nullptr);
+  const size_t split_bytes = p.split_s > 1 ? (size_t)p.split_tiles * p.split_s * p.bm * (128 + 1) * sizeof(float) : 0;
+  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && p.bm == 256 && ws_avail >= split_bytes + BOUND_WS_BYTES) {
+    ws_base += BOUND_WS_BYTES;
+    float* part = (float*)workspace;
+    int* flag = (int*)(part + 2 * BOUND_G);
+    const float limit = dtype == PA_DTYPE_BF16 ? 60.f : 14.f;
+    if (dtype == PA_DTYPE_BF16)
+      hipLaunchKernelGGL((score_bound_partial_kernel<BF16>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
+    else
+      hipLaunchKernelGGL((score_bound_partial_kernel<F16>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
+    PA_CHECK_LAUNCH("score bound kernel");
+    hipLaunchKernelGGL(score_bound_flag_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)part, p.scale_log2, limit, flag);
+    PA_CHECK_LAUNCH("score bound flag kernel");
+    p.bound_flag = flag;
+  }
   if (accumulate) {
     if (p.causal) PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation is not causal");
     if (!p.pipe || D != 128)  // only the head_dim-128 pipelined kernel has the folding epilogue
@@ -1990,7 +2126,7 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
     p.lse = nullptr;
   }
   if (p.split_s > 1) {
-    p.ws_out = (float*)workspace;
+    p.ws_out = (float*)ws_base;
     p.ws_lse = p.ws_out + (size_t)p.split_tiles * p.split_s * p.bm * 128;
   }
   return dispatch_attn<false>(p, dtype, D, (hipStream_t)stream);
@@ -2036,6 +2172,7 @@ extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int
   fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
   size_t need = 0;
   choose_kernel(p, D, 256, true, 0, &need);
+  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && p.bm == 256) need += BOUND_WS_BYTES;
   return need;
 }
 
