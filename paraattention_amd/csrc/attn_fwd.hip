@@ -1296,8 +1296,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
 // ---------------------------------------------------------------------------------------------
 constexpr int TILE64_BYTES = BN * 128;
 
-template <typename T, bool SPARSE, int NW>
+template <typename T, bool SPARSE, int NW, bool BOUNDED = false>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_kernel(const AttnParams p) {
+  // BOUNDED and the flag: as in attn_fwd_d128_pipe_kernel
+  if constexpr (!SPARSE) {
+    if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
+  }
   typedef typename T::vec8 vec8;
   constexpr int DC = 4, DB = 2;
   constexpr int IPW = 8 / NW;  // copy instructions per wavefront and K (V) tile
@@ -1403,7 +1407,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
   for (int i = 0; i < DB; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = BOUNDED ? 0.f : -INFINITY, l_run = 0.f;
   const float c = p.scale_log2;
 
   uint32_t n_cur, n_nxt, n_nx2;
@@ -1470,10 +1474,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
       else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
     }
     if (v_cur < BN || on_diagonal(n_cur)) mask_tail(sn0, sn1, v_cur, n_cur);
-    float m2 = fmaxf(sn0[0], sn1[0]);
+    if constexpr (!BOUNDED) {
+      float m2 = fmaxf(sn0[0], sn1[0]);
 #pragma unroll
-    for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
-    mx = across(m2);
+      for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
+      mx = across(m2);
+    }
   }
 
   auto tile_step = [&](auto PAR) {
@@ -1488,7 +1494,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
     for (int g = 0; g < 8; ++g) f[g] = read_k(tKn, g & 1, g >> 1);  // all of K(j+1), halves alternating
 
     const float mx_s = mx * c;
-    if (__any(mx_s > m_run + RESCALE_SLACK)) {
+    if (!BOUNDED && __any(mx_s > m_run + RESCALE_SLACK)) {
       const float m_new = fmaxf(m_run, mx_s);
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       l_run *= alpha;
@@ -1567,12 +1573,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
       for (int db = 0; db < DB; ++db) {
         const int g = 2 * cc + db;
         o[db] = T::mfma32(f[4 + g], bfrag, o[db]);
-        mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g]), sn0[4 * g + 1]), sn0[4 * g + 2]), sn0[4 * g + 3]);
-        mxb = fmaxf(fmaxf(fmaxf(fmaxf(mxb, sn1[4 * g]), sn1[4 * g + 1]), sn1[4 * g + 2]), sn1[4 * g + 3]);
+        if constexpr (!BOUNDED) {
+          mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g]), sn0[4 * g + 1]), sn0[4 * g + 2]), sn0[4 * g + 3]);
+          mxb = fmaxf(fmaxf(fmaxf(fmaxf(mxb, sn1[4 * g]), sn1[4 * g + 1]), sn1[4 * g + 2]), sn1[4 * g + 3]);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    mx = across(fmaxf(mxa, mxb));
+    if constexpr (!BOUNDED) mx = across(fmaxf(mxa, mxb));
 
     n_cur = n_nxt;
     v_cur = v_nxt;
@@ -1754,31 +1762,33 @@ __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int
 }
 
 // ---------------------------------------------------------------------------------------------
-// Score bound for the dense head_dim-128 kernel.  |q.k| <= |q| |k|, so with Mq = the largest row
+// Score bound for the dense pipelined kernels.  |q.k| <= |q| |k|, so with Mq = the largest row
 // norm of Q and Mk that of K no score leaves [-Mq Mk scale, Mq Mk scale]; in the log2 domain of the
 // kernel that is +-bound.  If bound <= `limit` (60 for bf16 P, whose exponent range is fp32's; 14
 // for fp16 P) then exp2(score) can neither overflow nor vanish, sums of up to 2^31 of them stay far
 // inside fp32, and the softmax needs no running maximum: a common factor 2^-m cancels in O / l and
 // in m + log2(l) whatever m is, so m = 0 gives the same results.  Models that normalise q and k
 // (RMS norm per head) sit near bound = 16.  Two launches: per-block maxima of the squared row
-// norms (blocks [0, G) over Q, [G, 2G) over K, 16 lanes per 256-byte row), then one block that
+// norms (blocks [0, G) over Q, [G, 2G) over K, 8 elements of a row per lane), then one block that
 // folds them and writes the flag.  An infinite element makes the bound infinite (flag 0); a NaN element
 // is not seen by the maxima, and its scores are NaN in either variant of the kernel.
 // ---------------------------------------------------------------------------------------------
 constexpr int BOUND_G = 1024;                                   // blocks per tensor
 constexpr size_t BOUND_WS_BYTES = (2 * BOUND_G + 64) * 4;       // partial maxima + the flag word (+ padding)
 
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnParams p, float* part) {
+  constexpr int LPR = D / 8;       // lanes per row: 8 elements each
+  constexpr int RPB = 256 / LPR;   // rows per block and step
   const bool is_k = blockIdx.x >= BOUND_G;
   const int blk = is_k ? blockIdx.x - BOUND_G : blockIdx.x;
   const uint16_t* base = (const uint16_t*)(is_k ? p.k : p.q);
   const int64_t sb = is_k ? p.ks_b : p.qs_b, sh = is_k ? p.ks_h : p.qs_h, ss = is_k ? p.ks_s : p.qs_s;
   const int S = is_k ? p.Skv : p.Sq;
   const int64_t rows = (int64_t)p.B * p.H * S;
-  const int sub = threadIdx.x & 15;
+  const int sub = threadIdx.x % LPR;
   float best = 0.f;
-  for (int64_t r = (int64_t)blk * 16 + (threadIdx.x >> 4); r < rows; r += (int64_t)BOUND_G * 16) {
+  for (int64_t r = (int64_t)blk * RPB + threadIdx.x / LPR; r < rows; r += (int64_t)BOUND_G * RPB) {
     const int s_ = (int)(r % S);
     const int64_t bh = r / S;
     const uint16_t* rp = base + (bh / p.H) * sb + (bh % p.H) * sh + (int64_t)s_ * ss + 8 * sub;
@@ -1791,7 +1801,7 @@ __global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnPara
       acc = __builtin_fmaf(b, b, acc);
     }
 #pragma unroll
-    for (int d = 1; d < 16; d <<= 1) acc += __shfl_xor(acc, d, 16);
+    for (int d = 1; d < LPR; d <<= 1) acc += __shfl_xor(acc, d, LPR);
     best = fmaxf(best, acc);
   }
   __shared__ float sm[256];
@@ -1905,24 +1915,32 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
     else { fn = (const void*)attn_fwd_kernel<T, D, SPARSE>; slot = 0; smem = Smem<D>::BYTES; }
   }
   // the attribute belongs to the function on one device: remembered per device and kernel variant
-  if (p.bound_flag != nullptr && !(D == 128 && slot == 2 && !SPARSE))
+  if (p.bound_flag != nullptr && (SPARSE || !(D == 128 ? slot == 2 : slot >= 1)))
     PA_FAIL(PA_ERR_UNSUPPORTED, "score bound reached a kernel that does not read it");
-  static bool attr_done[PA_MAX_DEVICES][4] = {};  // benign race: the call is idempotent
+  static bool attr_done[PA_MAX_DEVICES][5] = {};  // benign race: the call is idempotent
   const int dev = current_device();
   if (dev < 0 || !attr_done[dev][slot]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     if (dev >= 0) attr_done[dev][slot] = true;
   }
-  if constexpr (D == 128 && !SPARSE) {
+  if constexpr (!SPARSE) {
     if (p.bound_flag != nullptr) {  // the variant without a running maximum first; one of the two returns at once
-      const void* fb = (const void*)attn_fwd_d128_pipe_kernel<T, false, 8, true>;
-      if (dev < 0 || !attr_done[dev][3]) {
+      const void* fb;
+      if constexpr (D == 128) fb = (const void*)attn_fwd_d128_pipe_kernel<T, false, 8, true>;
+      else fb = slot == 2 ? (const void*)attn_fwd_d64_pipe_kernel<T, false, 8, true> : (const void*)attn_fwd_d64_pipe_kernel<T, false, 4, true>;
+      const int bslot = 3 + (D == 64 && slot == 1 ? 1 : 0);
+      if (dev < 0 || !attr_done[dev][bslot]) {
         hipError_t e = hipFuncSetAttribute(fb, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        if (dev >= 0) attr_done[dev][3] = true;
+        if (dev >= 0) attr_done[dev][bslot] = true;
       }
-      hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, false, 8, true>), dim3((unsigned)nblocks), dim3(512), smem, stream, p);
+      if constexpr (D == 128)
+        hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, false, 8, true>), dim3((unsigned)nblocks), dim3(512), smem, stream, p);
+      else if (slot == 2)
+        hipLaunchKernelGGL((attn_fwd_d64_pipe_kernel<T, false, 8, true>), dim3((unsigned)nblocks), dim3(512), smem, stream, p);
+      else
+        hipLaunchKernelGGL((attn_fwd_d64_pipe_kernel<T, false, 4, true>), dim3((unsigned)nblocks), dim3(256), smem, stream, p);
       PA_CHECK_LAUNCH("attention kernel (bounded scores)");
     }
   }
@@ -2068,14 +2086,16 @@ static int dispatch_attn(const AttnParams& p, int dtype, int D, hipStream_t stre
   return launch_attn<F16, 64, SPARSE>(p, stream);
 }
 
-// Whether a dense launch of this size is worth the two small launches that bound its scores (they read Q and K
-// once: about 45 us at the 119k-token shape, against 4 % of the attention kernel).  PARAATTN_BOUND=1 asks for the
-// bound at any size, =0 never (tuning and test aid).
+// Whether a dense launch of this size is worth the two small launches that bound its scores.  They read Q and K
+// once, the attention kernel gains 4 % (head_dim 128, 256 rows) to 6 % (head_dim 64): measured, the reads cost
+// 225..300 / S of the kernel's time at Sq = Skv = S (35 us against 17.6 ms at 119k tokens), so the sequences
+// must be long (Sq Skv / (Sq + Skv) >= 6144: 12k tokens) and the launch long enough to carry three more launch
+// gaps (1e12 flop).  PARAATTN_BOUND=1 asks for the bound at any size, =0 never (tuning and test aid).
 static bool bound_wanted(int B, int H, int Sq, int Skv, int D) {
-  if (D != 128 || B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0) return false;
+  if ((D != 128 && D != 64) || B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0) return false;
   if (env_is("PARAATTN_BOUND", "0")) return false;
   if (env_is("PARAATTN_BOUND", "1")) return true;
-  return 4.0 * B * H * (double)Sq * (double)Skv * D >= 2.0e12;
+  return (double)Sq * Skv >= 6144.0 * ((double)Sq + Skv) && 4.0 * B * H * (double)Sq * (double)Skv * D >= 1.0e12;
 }
 
 static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out, float* lse,
@@ -2104,15 +2124,19 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   char* ws_base = (char*)workspace;
   choose_kernel(p, D, 256, true, ws_avail, nullptr);
   const size_t split_bytes = p.split_s > 1 ? (size_t)p.split_tiles * p.split_s * p.bm * (128 + 1) * sizeof(float) : 0;
-  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && p.bm == 256 && ws_avail >= split_bytes + BOUND_WS_BYTES) {
+  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && (D == 64 || p.bm == 256) && ws_avail >= split_bytes + BOUND_WS_BYTES) {
     ws_base += BOUND_WS_BYTES;
     float* part = (float*)workspace;
     int* flag = (int*)(part + 2 * BOUND_G);
     const float limit = dtype == PA_DTYPE_BF16 ? 60.f : 14.f;
-    if (dtype == PA_DTYPE_BF16)
-      hipLaunchKernelGGL((score_bound_partial_kernel<BF16>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
+    if (dtype == PA_DTYPE_BF16 && D == 128)
+      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 128>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
+    else if (dtype == PA_DTYPE_BF16)
+      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 64>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
+    else if (D == 128)
+      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 128>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
     else
-      hipLaunchKernelGGL((score_bound_partial_kernel<F16>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
+      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 64>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
     PA_CHECK_LAUNCH("score bound kernel");
     hipLaunchKernelGGL(score_bound_flag_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)part, p.scale_log2, limit, flag);
     PA_CHECK_LAUNCH("score bound flag kernel");
@@ -2166,13 +2190,13 @@ extern "C" int pa_attn_fwd_accumulate(const void* q, const void* k, const void* 
 
 extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
                                               const int64_t k_strides[3], const int64_t v_strides[3]) {
-  if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D != 128 || !k_strides || !v_strides) return 0;
+  if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || (D != 128 && D != 64) || !k_strides || !v_strides) return 0;
   AttnParams p;
   const int64_t zero[3] = {0, 0, 0};
   fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
   size_t need = 0;
   choose_kernel(p, D, 256, true, 0, &need);
-  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && p.bm == 256) need += BOUND_WS_BYTES;
+  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && (D == 64 || p.bm == 256)) need += BOUND_WS_BYTES;
   return need;
 }
 

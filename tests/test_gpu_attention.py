@@ -280,14 +280,16 @@ def test_key_split_tail(cuda, bm, monkeypatch):
     monkeypatch.delenv("PARAATTN_BM")
 
 
+@pytest.mark.parametrize("D,bm", [(128, "256"), (64, "128"), (64, "256")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_score_bound_variants(cuda, dtype, monkeypatch):
-    """The 256-row kernel drops the running maximum when |q| |k| scale bounds every score (computed on the device);
-    forced on at a small size here.  Unit-variance inputs sit below the bf16 limit (bound about 23 of 60) and above
-    the fp16 one (14); inputs four times larger exceed both, so both variants run for each type or shape; every case
-    is checked against the fp64 oracle and against the launch without the bound."""
-    monkeypatch.setenv("PARAATTN_BM", "256")
-    B, H, Sq, Skv, D = 2, 3, 700, 1500, 128
+def test_score_bound_variants(cuda, dtype, D, bm, monkeypatch):
+    """The dense kernels (head_dim 128: 256 rows; head_dim 64: both sizes) drop the running maximum when
+    |q| |k| scale bounds every score (computed on the device); forced on at a small size here.  Unit-variance inputs
+    sit below the bf16 limit (bound about 23 of 60) and above the fp16 one (14); inputs four times larger exceed
+    both, smaller ones neither, so both variants run for each type; every case is checked against the fp64 oracle
+    and against the launch without the bound."""
+    monkeypatch.setenv("PARAATTN_BM", bm)
+    B, H, Sq, Skv = 2, 3, 700, 1500
     op = torch.ops.para_attn.attention_forward_with_lse
     for gain, kgain in ((1.0, 1.0), (4.0, 4.0), (0.25, 1.0), (1.0, 0.0)):
         q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=31, dtype=dtype)
