@@ -26,7 +26,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM-side traffic per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two rocprofv3 --pmc
 # runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy; the summaries are kept under profiles/)
-TRAFFIC = {"attn": 4.192e9, "merge": 4.629e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 2.038e10}
+TRAFFIC = {"attn": 4.136e9, "merge": 4.632e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 1.931e10}
 
 
 def _time_calls(fn, steps, warmup):
