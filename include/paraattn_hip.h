@@ -47,6 +47,21 @@ PA_API int pa_abi_version(void);
 PA_API const char* pa_last_error(void);
 
 /*
+ * Tuning and test aids of the attention launches (no counterpart in the
+ * reference, whose aten kernels choose their own variants).  Each knob starts
+ * from an environment variable that is read once per process, at the first
+ * launch; this call changes it afterwards, for all later launches of the
+ * process:
+ *   "no_pipe"      PARAATTN_NO_PIPE=1       1: the kernels without 32-bit offset limits
+ *   "bm"           PARAATTN_BM=128|256      query rows per workgroup, 0 = chosen per launch
+ *   "no_split"     PARAATTN_NO_SPLIT=1      1: no key-split tail
+ *   "no_xcd_order" PARAATTN_NO_XCD_ORDER=1  1: block-sparse workgroups in plain order
+ *   "bound"        PARAATTN_BOUND=0|1       0 / 1: never / always compute the score bound, -1 = by size
+ * Returns PA_ERR_INVALID for an unknown name or value.
+ */
+PA_API int pa_set_tuning(const char* name, int value);
+
+/*
  * Dense scaled-dot-product attention forward.
  *   out[b,h,i,:] = softmax_j(scale * q[b,h,i,:].k[b,h,j,:]) @ v[b,h,j,:]
  *   lse[b,h,i]   = log sum_j exp(scale * q.k)      (natural log, fp32)

@@ -22,7 +22,7 @@ PA_DTYPE_BF16 = 0
 PA_DTYPE_F16 = 1
 PA_DTYPE_F32 = 2
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -37,6 +37,7 @@ _floats = ctypes.POINTER(ctypes.c_float)  # host array
 SIGNATURES = {
     "pa_abi_version": (_i, []),
     "pa_last_error": (ctypes.c_char_p, []),
+    "pa_set_tuning": (_i, [ctypes.c_char_p, _i]),
     "pa_attn_fwd_lse": (
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _i, _vp],
@@ -115,6 +116,12 @@ def check(rc, what):
     if rc == PA_ERR_INVALID:
         raise ValueError(text)
     raise HipLibraryError(text)
+
+
+def set_tuning(name, value):
+    """Set one tuning / test knob of the attention launches (pa_set_tuning in the header): "no_pipe", "bm",
+    "no_split", "no_xcd_order", "bound".  The PARAATTN_* environment variables only give the initial values."""
+    check(load().pa_set_tuning(name.encode(), int(value)), "pa_set_tuning")
 
 
 def strides3(t):

@@ -29,6 +29,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "pa_common.h"
@@ -2005,9 +2006,47 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
   return found;
 }
 
-static bool env_is(const char* name, const char* val) {
-  const char* e = getenv(name);
-  return e && strcmp(e, val) == 0;
+// Tuning and test aids.  The environment gives the initial values and is read once per process
+// (at the first launch); pa_set_tuning() changes them afterwards.
+//   PARAATTN_NO_PIPE=1       "no_pipe"       the kernels without 32-bit offset limits
+//   PARAATTN_BM=128|256      "bm"            query rows per workgroup (0 = choose)
+//   PARAATTN_NO_SPLIT=1      "no_split"      no key-split tail
+//   PARAATTN_NO_XCD_ORDER=1  "no_xcd_order"  block-sparse workgroups in plain order
+//   PARAATTN_BOUND=0|1       "bound"         never / always compute the score bound (-1 = by size)
+struct Tuning {
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound;
+};
+static Tuning& tuning() {
+  static Tuning t;
+  static const bool init = [] {
+    auto num = [](const char* name, int dflt) {
+      const char* e = getenv(name);
+      return e && *e ? atoi(e) : dflt;
+    };
+    t.no_pipe = num("PARAATTN_NO_PIPE", 0) == 1;
+    t.no_split = num("PARAATTN_NO_SPLIT", 0) == 1;
+    t.no_xcd_order = num("PARAATTN_NO_XCD_ORDER", 0) == 1;
+    t.forced_bm = num("PARAATTN_BM", 0);
+    const int b = num("PARAATTN_BOUND", -1);
+    t.bound = b == 0 || b == 1 ? b : -1;
+    return true;
+  }();
+  (void)init;
+  return t;
+}
+
+extern "C" int pa_set_tuning(const char* name, int value) {
+  if (!name) PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: null name");
+  Tuning& t = tuning();
+  if (!strcmp(name, "no_pipe")) t.no_pipe = value == 1;
+  else if (!strcmp(name, "no_split")) t.no_split = value == 1;
+  else if (!strcmp(name, "no_xcd_order")) t.no_xcd_order = value == 1;
+  else if (!strcmp(name, "bm")) {
+    if (value != 0 && value != 128 && value != 256) PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: bm must be 0, 128 or 256");
+    t.forced_bm = value;
+  } else if (!strcmp(name, "bound")) t.bound = value == 0 || value == 1 ? value : -1;
+  else PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: unknown knob '%s'", name);
+  return PA_OK;
 }
 
 // Bytes of workspace the key-split tail of the plan for bm rows per workgroup needs.
@@ -2032,10 +2071,9 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
   if (p.Skv <= 0 || (uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB ||
       (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB)
     return finish();
-  if (env_is("PARAATTN_NO_PIPE", "1")) return finish();  // test aid: the kernels without offset limits
+  if (tuning().no_pipe) return finish();  // test aid: the kernels without offset limits
   p.pipe = 1;
-  const char* force = getenv("PARAATTN_BM");  // tuning aid
-  const int forced = force ? atoi(force) : 0;
+  const int forced = tuning().forced_bm;  // tuning aid
   if (D == 64) {  // no key split at head_dim 64; 128 rows unless asked otherwise
     if (forced == 256 && (dense || q_block % 256 == 0)) p.bm = 256;
     return finish();
@@ -2046,7 +2084,7 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
   }
   const int cus = device_cus();
   // (causal workgroups differ in length: the rounds estimate does not apply, no split)
-  const bool allow = cus > 0 && !p.causal && !env_is("PARAATTN_NO_SPLIT", "1") && (ws_needed != nullptr || ws_bytes > 0);
+  const bool allow = cus > 0 && !p.causal && !tuning().no_split && (ws_needed != nullptr || ws_bytes > 0);
   const int kv_tiles = (p.Skv + BN - 1) / BN;
   const int64_t bh = (int64_t)p.B * p.H;
   const int64_t n128 = bh * ((p.Sq + 127) / 128), n256 = bh * ((p.Sq + 255) / 256);
@@ -2093,8 +2131,7 @@ static int dispatch_attn(const AttnParams& p, int dtype, int D, hipStream_t stre
 // gaps (1e12 flop).  PARAATTN_BOUND=1 asks for the bound at any size, =0 never (tuning and test aid).
 static bool bound_wanted(int B, int H, int Sq, int Skv, int D) {
   if ((D != 128 && D != 64) || B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0) return false;
-  if (env_is("PARAATTN_BOUND", "0")) return false;
-  if (env_is("PARAATTN_BOUND", "1")) return true;
+  if (tuning().bound >= 0) return tuning().bound == 1;
   return (double)Sq * Skv >= 6144.0 * ((double)Sq + Skv) && 4.0 * B * H * (double)Sq * (double)Skv * D >= 1.0e12;
 }
 
@@ -2251,7 +2288,7 @@ extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void*
   const int q_hi = q_lo + nQ * q_block;
   const int tiles_right = (Sq - q_hi + p.bm - 1) / p.bm;
   p.n_qtiles = p.tiles_left + nQ * p.tiles_per_block + tiles_right;
-  if (D == 128 && p.pipe && !env_is("PARAATTN_NO_XCD_ORDER", "1"))
+  if (D == 128 && p.pipe && !tuning().no_xcd_order)
     p.xcd_chunk = (int)(((int64_t)B * H * p.n_qtiles + 7) / 8);
   return dispatch_attn<true>(p, dtype, D, (hipStream_t)stream);
 }

@@ -7,9 +7,7 @@ reference's adapters swap in for a model's block list (utils.py:333-451).  The
 diffusers adapters themselves are not part of this package.
 """
 import contextlib
-import dataclasses
-from collections import defaultdict
-from typing import Any, DefaultDict, Dict, List, Optional, Union
+import itertools
 
 import torch
 
@@ -17,98 +15,62 @@ from . import ops
 from .taylorseer import TaylorSeer
 
 
-@dataclasses.dataclass
+class _Lane:
+    """What one of the two passes of a step owns: its buffers, its TaylorSeer, its threshold.  A
+    pipeline without an alternating pass (classifier-free guidance run as a second forward) only
+    ever uses the main lane."""
+
+    __slots__ = ("suffix", "threshold", "store", "seer")
+
+    def __init__(self, suffix, threshold, seer):
+        self.suffix = suffix
+        self.threshold = threshold
+        self.store = {}
+        self.seer = seer
+
+
+def _as_float(x):
+    return x.item() if isinstance(x, torch.Tensor) else x
+
+
 class CacheContext:
-    """State of one pipeline call (reference fields of the same names, utils.py:12-37)."""
+    """State of one pipeline call.  Constructor arguments are the reference's fields of the same
+    names and order (src/para_attn/first_block_cache/utils.py:12-28); the bookkeeping is kept as one
+    count of ``mark_step_begin`` calls, from which the running step and the pass (main or
+    alternating) follow, and one lane of buffers per pass.
 
-    residual_diff_threshold: Union[torch.Tensor, float] = 0.0
-    alter_residual_diff_threshold: Optional[Union[torch.Tensor, float]] = None
-    downsample_factor: int = 1
-    enable_alter_cache: bool = False
-    num_inference_steps: int = -1
-    warmup_steps: int = 0
-    enable_taylorseer: bool = False
-    taylorseer_kwargs: Dict[str, Any] = dataclasses.field(default_factory=dict)
-    slg_layers: Optional[List[int]] = None
-    slg_start: float = 0.0
-    slg_end: float = 0.1
-    taylorseer: Optional[TaylorSeer] = None
-    alter_taylorseer: Optional[TaylorSeer] = None
-    buffers: Dict[str, Any] = dataclasses.field(default_factory=dict)
-    incremental_name_counters: DefaultDict[str, int] = dataclasses.field(default_factory=lambda: defaultdict(int))
-    executed_steps: int = 0
-    is_alter_cache: bool = True
+    With ``enable_alter_cache`` the calls alternate main, alter, main, ... and a step is one such
+    pair; before the first call the context stands on the alternating pass (utils.py:37, 80-88).
+    Without it every call is a step of the main pass.
+    """
 
-    def __post_init__(self):
-        if self.enable_taylorseer:
-            self.taylorseer = TaylorSeer(**self.taylorseer_kwargs)
-            if self.enable_alter_cache:
-                self.alter_taylorseer = TaylorSeer(**self.taylorseer_kwargs)
+    def __init__(self, residual_diff_threshold=0.0, alter_residual_diff_threshold=None, downsample_factor=1,
+                 enable_alter_cache=False, num_inference_steps=-1, warmup_steps=0, enable_taylorseer=False,
+                 taylorseer_kwargs=None, slg_layers=None, slg_start=0.0, slg_end=0.1):
+        self.downsample_factor = downsample_factor
+        self.enable_alter_cache = enable_alter_cache
+        self.num_inference_steps = num_inference_steps
+        self.warmup_steps = warmup_steps
+        self.enable_taylorseer = enable_taylorseer
+        self.taylorseer_kwargs = dict(taylorseer_kwargs or {})
+        self.slg_layers = slg_layers
+        self.slg_start = slg_start
+        self.slg_end = slg_end
+        seer = lambda wanted: TaylorSeer(**self.taylorseer_kwargs) if wanted else None  # noqa: E731
+        self._main = _Lane("", residual_diff_threshold, seer(enable_taylorseer))
+        self._alter = _Lane("_alter", alter_residual_diff_threshold, seer(enable_taylorseer and enable_alter_cache))
+        self._marks = 0        # mark_step_begin calls so far
+        self._serials = {}     # name -> iterator of its serial numbers
 
-    def get_incremental_name(self, name=None):
-        """utils.py:45-50: "<name>_<count>", counting per name from 0."""
-        name = "default" if name is None else name
-        idx = self.incremental_name_counters[name]
-        self.incremental_name_counters[name] += 1
-        return f"{name}_{idx}"
+    # -- where the context stands --------------------------------------------------------------------
+    @property
+    def is_alter_cache(self):
+        """True on the alternating pass; stays True when there is none (the reference's flag, utils.py:37)."""
+        return not self.enable_alter_cache or self._marks % 2 == 0
 
-    def reset_incremental_names(self):
-        self.incremental_name_counters.clear()
-
-    def get_taylorseer(self):
-        if self.enable_alter_cache and self.is_alter_cache:
-            return self.alter_taylorseer
-        return self.taylorseer
-
-    def get_residual_diff_threshold(self):
-        if self.enable_alter_cache and self.is_alter_cache and self.alter_residual_diff_threshold is not None:
-            thr = self.alter_residual_diff_threshold
-        else:
-            thr = self.residual_diff_threshold
-        if isinstance(thr, torch.Tensor):
-            thr = thr.item()
-        return thr
-
-    def _name(self, name):
-        return f"{name}_alter" if self.enable_alter_cache and self.is_alter_cache else name
-
-    def get_buffer(self, name):
-        return self.buffers.get(self._name(name))
-
-    def set_buffer(self, name, buffer):
-        self.buffers[self._name(name)] = buffer
-
-    def remove_buffer(self, name):
-        self.buffers.pop(self._name(name), None)
-
-    def clear_buffers(self):
-        self.buffers.clear()
-
-    def mark_step_begin(self):
-        if not self.enable_alter_cache:
-            self.executed_steps += 1
-        else:
-            self.is_alter_cache = not self.is_alter_cache
-            if not self.is_alter_cache:
-                self.executed_steps += 1
-        if self.enable_taylorseer:
-            self.get_taylorseer().mark_step_begin()
-
-    def is_slg_enabled(self):
-        return self.slg_layers is not None
-
-    def slg_should_skip_block(self, block_idx):
-        """utils.py:102-114: skip-layer guidance drops the listed blocks on the alternating pass, inside
-        the step window [slg_start, slg_end) of the schedule."""
-        if not self.enable_alter_cache or not self.is_alter_cache:
-            return False
-        if self.slg_layers is None:
-            return False
-        if self.slg_start <= 0.0 and self.slg_end >= 1.0:
-            return False
-        assert self.num_inference_steps >= 0, "num_inference_steps must be non-negative"
-        n = self.num_inference_steps
-        return block_idx in self.slg_layers and n * self.slg_start <= self.get_current_step() < n * self.slg_end
+    @property
+    def executed_steps(self):
+        return (self._marks + 1) // 2 if self.enable_alter_cache else self._marks
 
     def get_current_step(self):
         return self.executed_steps - 1
@@ -116,8 +78,90 @@ class CacheContext:
     def is_in_warmup(self):
         return self.get_current_step() < self.warmup_steps
 
+    def _lane(self):
+        return self._alter if self.enable_alter_cache and self._marks % 2 == 0 else self._main
 
-_current_cache_context = None
+    def mark_step_begin(self):
+        """One forward pass of the model begins (utils.py:80-90)."""
+        self._marks += 1
+        seer = self._lane().seer
+        if seer is not None:
+            seer.mark_step_begin()
+
+    # -- per-pass settings -----------------------------------------------------------------------------
+    @property
+    def residual_diff_threshold(self):
+        return self._main.threshold
+
+    @property
+    def alter_residual_diff_threshold(self):
+        return self._alter.threshold
+
+    def get_residual_diff_threshold(self):
+        """Python number; the alternating pass has its own if one was given (utils.py:55-62)."""
+        own = self._lane().threshold
+        return _as_float(self._main.threshold if own is None else own)
+
+    @property
+    def taylorseer(self):
+        return self._main.seer
+
+    @property
+    def alter_taylorseer(self):
+        return self._alter.seer
+
+    def get_taylorseer(self):
+        return self._lane().seer
+
+    # -- buffers ----------------------------------------------------------------------------------------
+    def get_buffer(self, name):
+        return self._lane().store.get(name)
+
+    def set_buffer(self, name, buffer):
+        self._lane().store[name] = buffer
+
+    def remove_buffer(self, name):
+        self._lane().store.pop(name, None)
+
+    def clear_buffers(self):
+        self._main.store.clear()
+        self._alter.store.clear()
+
+    @property
+    def buffers(self):
+        """All buffers under the reference's names: those of the alternating pass carry "_alter" (utils.py:64-72)."""
+        return {name + lane.suffix: buf for lane in (self._main, self._alter) for name, buf in lane.store.items()}
+
+    # -- serial names -----------------------------------------------------------------------------------
+    def get_incremental_name(self, name=None):
+        """"<name>_<n>" with n = 0, 1, ... per name (utils.py:45-50)."""
+        stem = "default" if name is None else name
+        return f"{stem}_{next(self._serials.setdefault(stem, itertools.count()))}"
+
+    def reset_incremental_names(self):
+        self._serials = {}
+
+    # -- skip-layer guidance ------------------------------------------------------------------------------
+    def is_slg_enabled(self):
+        return self.slg_layers is not None
+
+    def slg_should_skip_block(self, block_idx):
+        """Skip-layer guidance (utils.py:102-114) drops the listed blocks on the alternating pass while
+        the running step lies in [slg_start, slg_end) of the schedule; a window that covers the whole
+        schedule switches it off."""
+        if not (self.enable_alter_cache and self._marks % 2 == 0) or self.slg_layers is None:
+            return False
+        if self.slg_start <= 0.0 and self.slg_end >= 1.0:
+            return False
+        assert self.num_inference_steps >= 0, "num_inference_steps must be non-negative"
+        lo, hi = self.num_inference_steps * self.slg_start, self.num_inference_steps * self.slg_end
+        return lo <= self.get_current_step() < hi and block_idx in self.slg_layers
+
+
+# The context in force, innermost last.  set_current_cache_context() replaces the innermost one,
+# cache_context() nests (src/para_attn/first_block_cache/utils.py:193-217: one module-wide context,
+# not per thread).
+_contexts = [None]
 
 
 def create_cache_context(*args, **kwargs):
@@ -125,23 +169,20 @@ def create_cache_context(*args, **kwargs):
 
 
 def get_current_cache_context():
-    return _current_cache_context
+    return _contexts[-1]
 
 
 def set_current_cache_context(cache_context=None):
-    global _current_cache_context
-    _current_cache_context = cache_context
+    _contexts[-1] = cache_context
 
 
 @contextlib.contextmanager
 def cache_context(cache_context):
-    global _current_cache_context
-    old = _current_cache_context
-    _current_cache_context = cache_context
+    _contexts.append(cache_context)
     try:
         yield
     finally:
-        _current_cache_context = old
+        _contexts.pop()
 
 
 def _ctx():

@@ -6,6 +6,7 @@ import torch
 import torch.nn.functional as F
 
 from . import ops
+from .interface import _SdpaMode
 
 
 def struct_sparse_attn_func(
@@ -53,24 +54,20 @@ def struct_sparse_attn_func(
     return out
 
 
-class StructSparseAttnMode(torch.overrides.TorchFunctionMode):
+class StructSparseAttnMode(_SdpaMode):
     """Reroutes ``F.scaled_dot_product_attention`` to the block-sparse kernel while active
-    (the reference's mode of the same name, src/para_attn/sparse_attn.py:643-693)."""
+    (the reference's mode of the same name, src/para_attn/sparse_attn.py:643-693), with the class-wide
+    ``disabled`` switch and ``disable()`` context of the other modes (:679-692)."""
 
-    def __init__(self, *, sparse_mask=None, sparse_range_query=None, sparse_range_key_value=None):
+    disabled = False
+
+    @torch.compiler.disable
+    def __init__(self, *, sparse_mask=None, sparse_range_query=None, sparse_range_key_value=None,
+                 print_attn_weight_means=False):
         super().__init__()
-        self._sparse_mask = sparse_mask
-        self._sparse_range_query = sparse_range_query
-        self._sparse_range_key_value = sparse_range_key_value
+        self._sparse = dict(sparse_mask=sparse_mask, sparse_range_query=sparse_range_query,
+                            sparse_range_key_value=sparse_range_key_value,
+                            print_attn_weight_means=print_attn_weight_means)
 
-    def __torch_function__(self, func, types, args=(), kwargs=None):
-        kwargs = {} if kwargs is None else kwargs
-        if func is F.scaled_dot_product_attention:
-            return struct_sparse_attn_func(
-                *args,
-                **kwargs,
-                sparse_mask=self._sparse_mask,
-                sparse_range_query=self._sparse_range_query,
-                sparse_range_key_value=self._sparse_range_key_value,
-            )
-        return func(*args, **kwargs)
+    def _call(self, *args, **kwargs):
+        return struct_sparse_attn_func(*args, **kwargs, **self._sparse)

@@ -19,3 +19,16 @@ def cuda():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+_KNOB_DEFAULTS = {"no_pipe": 0, "bm": 0, "no_split": 0, "no_xcd_order": 0, "bound": -1}
+
+
+@pytest.fixture
+def tuning():
+    """Setter for the library's tuning knobs (pa_set_tuning); every knob is back at its default after the test."""
+    from paraattention_amd import _lib
+
+    yield _lib.set_tuning
+    for name, val in _KNOB_DEFAULTS.items():
+        _lib.set_tuning(name, val)

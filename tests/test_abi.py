@@ -94,6 +94,22 @@ def test_argument_validation_without_device_work():
     assert lib.pa_fbcache_apply_residual(a, a, a, 0, 0, None) == _lib.PA_OK
 
 
+def test_tuning_knobs_are_validated():
+    lib = _lib.load()
+    try:
+        assert lib.pa_set_tuning(b"bm", 256) == _lib.PA_OK
+        assert lib.pa_set_tuning(b"bm", 100) == _lib.PA_ERR_INVALID and b"bm" in lib.pa_last_error()
+        assert lib.pa_set_tuning(b"no_such_knob", 1) == _lib.PA_ERR_INVALID
+        assert lib.pa_set_tuning(None, 1) == _lib.PA_ERR_INVALID
+        for name in (b"no_pipe", b"no_split", b"no_xcd_order", b"bound"):
+            assert lib.pa_set_tuning(name, 1) == _lib.PA_OK
+        with pytest.raises(ValueError):
+            _lib.set_tuning("bm", 64)
+    finally:
+        for name, val in (("no_pipe", 0), ("bm", 0), ("no_split", 0), ("no_xcd_order", 0), ("bound", -1)):
+            _lib.set_tuning(name, val)
+
+
 def test_missing_library_is_loud():
     code = "import paraattention_amd._lib as l\ntry:\n    l.load()\nexcept ImportError as e:\n    print('IMPORTERROR', 'no CPU or eager fallback' in str(e))\n"
     env = dict(os.environ, PARAATTN_HIP_LIB="/nonexistent/libparaattn_hip.so", PYTHONPATH=ROOT)

@@ -204,27 +204,25 @@ def test_empty_inputs(cuda, D):
     assert out.shape == (2, 2, 0, D) and lse.shape == (2, 2, 0)
 
 
-@pytest.mark.parametrize("env", [{"PARAATTN_NO_PIPE": "1"}, {"PARAATTN_BM": "256"}])
-def test_alternative_kernels(cuda, env, monkeypatch):
+@pytest.mark.parametrize("env", [{"no_pipe": 1}, {"bm": 256}])
+def test_alternative_kernels(cuda, env, tuning):
     """The kernels without 32-bit offset limits (taken when K or V spans 4 GiB or more) and the 8-wavefront
     workgroup variants compute the same thing as the default kernels, at head_dim 128 and 64."""
-    import os
-
     cases = [(1, 2, 300, 434, 128), (2, 1, 129, 1000, 128), (1, 1, 64, 64, 128), (1, 3, 1000, 77, 128),
              (1, 2, 300, 434, 64), (2, 1, 129, 1000, 64), (1, 3, 1000, 77, 64)]
     for B, H, Sq, Skv, D in cases:
         q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=Sq + Skv)
         ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
         for name, val in env.items():
-            monkeypatch.setenv(name, val)
+            tuning(name, val)
         out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
         for name in env:
-            monkeypatch.delenv(name)
+            tuning(name, 0)
         _check(out, lse, ref_out, ref_lse, f"{env} {(B, H, Sq, Skv)}")
 
 
 @pytest.mark.parametrize("bm", ["128", "256"])
-def test_key_split_tail(cuda, bm, monkeypatch):
+def test_key_split_tail(cuda, bm, tuning):
     """Grids a little over a whole number of rounds: the query tiles of the last round are computed in key
     shares (fp32 partials in a workspace) and merged.  Checked against the oracle, against the unsplit launch,
     with per-batch key counts that leave some shares empty, and with a strided output."""
@@ -240,17 +238,17 @@ def test_key_split_tail(cuda, bm, monkeypatch):
     Skv = 64 * 40 + 37
     q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=77)
     qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
-    monkeypatch.setenv("PARAATTN_BM", bm)
+    tuning("bm", int(bm))
     need = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, _lib.strides3(kd), _lib.strides3(vd))
     assert need > 0, "this shape is meant to take the key-split path"
     ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q, k, v)
     out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd)
     _check(out, lse, ref_out.float().numpy(), ref_lse.numpy(), f"split bm={bm}")
-    monkeypatch.setenv("PARAATTN_NO_SPLIT", "1")
+    tuning("no_split", 1)
     # no partials any more (what remains, if the score bound is asked for at this size, is its 8 KB)
     assert lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, _lib.strides3(kd), _lib.strides3(vd)) < 16384
     out1, lse1 = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd)
-    monkeypatch.delenv("PARAATTN_NO_SPLIT")
+    tuning("no_split", 0)
     assert (out.float() - out1.float()).abs().max().item() <= 2e-2
     assert (lse - lse1).abs().max().item() <= 1e-4
     # a workspace that is too short is not an error: the launch is the unsplit one
@@ -277,32 +275,29 @@ def test_key_split_tail(cuda, bm, monkeypatch):
     qs = qd.transpose(1, 2).contiguous().transpose(1, 2)
     out2, lse2 = torch.ops.para_attn.attention_forward_with_lse(qs, kd, vd, keep[:, None, None, :].to(cuda))
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
-    monkeypatch.delenv("PARAATTN_BM")
 
 
 @pytest.mark.parametrize("D,bm", [(128, "256"), (64, "128"), (64, "256")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_score_bound_variants(cuda, dtype, D, bm, monkeypatch):
+def test_score_bound_variants(cuda, dtype, D, bm, tuning):
     """The dense kernels (head_dim 128: 256 rows; head_dim 64: both sizes) drop the running maximum when
     |q| |k| scale bounds every score (computed on the device); forced on at a small size here.  Unit-variance inputs
     sit below the bf16 limit (bound about 23 of 60) and above the fp16 one (14); inputs four times larger exceed
     both, smaller ones neither, so both variants run for each type; every case is checked against the fp64 oracle
     and against the launch without the bound."""
-    monkeypatch.setenv("PARAATTN_BM", bm)
+    tuning("bm", int(bm))
     B, H, Sq, Skv = 2, 3, 700, 1500
     op = torch.ops.para_attn.attention_forward_with_lse
     for gain, kgain in ((1.0, 1.0), (4.0, 4.0), (0.25, 1.0), (1.0, 0.0)):
         q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=31, dtype=dtype)
         q, k = (q.float() * gain).to(dtype), (k.float() * kgain).to(dtype)
         ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
-        monkeypatch.setenv("PARAATTN_BOUND", "1")
+        tuning("bound", 1)
         out, lse = op(q.to(cuda), k.to(cuda), v.to(cuda))
         _check(out, lse, ref_out, ref_lse, f"bound on, gain {gain} {kgain} {dtype}")
-        monkeypatch.setenv("PARAATTN_BOUND", "0")
+        tuning("bound", 0)
         out0, lse0 = op(q.to(cuda), k.to(cuda), v.to(cuda))
         assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
-    monkeypatch.delenv("PARAATTN_BOUND")
-    monkeypatch.delenv("PARAATTN_BM")
 
 
 CAUSAL = [(1, 2, 1, 1), (1, 1, 17, 17), (2, 2, 64, 64), (1, 2, 129, 129), (1, 1, 300, 300), (1, 2, 700, 700),
@@ -322,17 +317,17 @@ def test_causal_vs_f64(cuda, B, H, Sq, Skv, D):
     assert torch.equal(torch.ops.para_attn.attention_forward(qd, kd, vd, is_causal=True), out)
 
 
-@pytest.mark.parametrize("env", [{"PARAATTN_NO_PIPE": "1"}, {"PARAATTN_BM": "256"}, {"PARAATTN_BM": "128"}])
-def test_causal_alternative_kernels(cuda, env, monkeypatch):
+@pytest.mark.parametrize("env", [{"no_pipe": 1}, {"bm": 256}, {"bm": 128}])
+def test_causal_alternative_kernels(cuda, env, tuning):
     for B, H, Sq, Skv, D in [(1, 2, 700, 700, 128), (1, 1, 300, 90, 128), (1, 2, 90, 300, 128), (2, 1, 513, 513, 128),
                              (1, 2, 700, 700, 64), (1, 1, 300, 90, 64), (2, 1, 513, 513, 64)]:
         q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=Sq + Skv)
         ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, oattn.causal_keep(Sq, Skv))
         for name, val in env.items():
-            monkeypatch.setenv(name, val)
+            tuning(name, val)
         out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), is_causal=True)
         for name in env:
-            monkeypatch.delenv(name)
+            tuning(name, 0)
         _check(out, lse, ref_out, ref_lse, f"causal {env} {(B, H, Sq, Skv, D)}")
 
 

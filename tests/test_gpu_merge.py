@@ -44,6 +44,31 @@ def test_merge_step_vs_oracle(cuda, shape, blk_dtype):
     assert lse4.shape == (B, H, S, 1) and torch.equal(out4, out)
 
 
+@pytest.mark.parametrize("D", [24, 48, 72, 80, 200])
+@pytest.mark.parametrize("acc_dtype", [torch.float32, torch.bfloat16])
+def test_merge_in_place_head_dims_off_the_wavefront(cuda, D, acc_dtype):
+    """In-place steps at head dims whose 8-element chunk count does not divide 64: a row's threads then straddle
+    wavefronts (D = 48: rows 10, 21 ... start in one wavefront and end in the next), and the step must still read
+    the old LSE for every chunk.  Many rows, so that every position of a row inside a wavefront and a workgroup
+    occurs; checked against the oracle's step and bit for bit against the functional op, which never aliases."""
+    B, H, S = 2, 3, 1777
+    o1, l1, o2, l2 = _partials(B, H, S, D, seed=D, dtype=acc_dtype)
+    # weights far from 0 and 1 on most rows, so an element merged with the new LSE instead of the old one shows
+    ref_out, ref_lse = omerge.merge_step(o1.float().numpy(), l1.numpy(), o2.float().numpy(), l2.numpy())
+    want, want_l = torch.ops.para_attn.merge_attention_lse(o1.to(cuda), l1.to(cuda), o2.to(cuda), l2.to(cuda), acc_dtype)
+    acc, acc_l = o1.to(cuda), l1.clone().to(cuda)
+    torch.ops.para_attn.merge_attention_lse_(acc, acc_l, o2.to(cuda), l2.to(cuda))
+    assert torch.equal(acc, want) and torch.equal(acc_l, want_l)
+    tol = dict(rtol=1e-5, atol=1e-5) if acc_dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-5)
+    np.testing.assert_allclose(acc.float().cpu().numpy(), ref_out, **tol)
+    np.testing.assert_allclose(acc_l.cpu().numpy(), ref_lse, rtol=1e-6, atol=2e-6)
+    # a second step on the merged pair (the accumulator's LSE now differs from row to row in the last bits)
+    o3, l3, _, _ = _partials(B, H, S, D, seed=D + 1, dtype=acc_dtype)
+    want2, want_l2 = torch.ops.para_attn.merge_attention_lse(acc.clone(), acc_l.clone(), o3.to(cuda), l3.to(cuda), acc_dtype)
+    torch.ops.para_attn.merge_attention_lse_(acc, acc_l, o3.to(cuda), l3.to(cuda))
+    assert torch.equal(acc, want2) and torch.equal(acc_l, want_l2)
+
+
 def test_merge_vs_torch_sdpa_merger(cuda):
     from torch.distributed.tensor.experimental._context_parallel._attention import _SDPAMerger
 
@@ -87,7 +112,7 @@ def test_ring_sweep_equals_full_attention(cuda, fused):
     np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
 
 
-def test_fused_accumulate_steps(cuda, monkeypatch):
+def test_fused_accumulate_steps(cuda, tuning):
     """attention_forward_accumulate_ / _final against the oracle's merge of the oracle's partials, on a grid that
     takes the key-split tail (so the split merge folds the accumulator too), with a strided query."""
     from oracle import merge as omerge
@@ -117,7 +142,7 @@ def test_fused_accumulate_steps(cuda, monkeypatch):
     np.testing.assert_allclose(acc_l[:, :, rows].cpu().numpy(), ref_lse, atol=1e-3)
     np.testing.assert_allclose(out[:, :, rows].float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
     # unsplit launch gives the same (to rounding)
-    monkeypatch.setenv("PARAATTN_NO_SPLIT", "1")
+    tuning("no_split", 1)
     acc_l2 = acc_l.clone()
     torch.ops.para_attn.attention_forward_accumulate_(acc, acc_l2, qd, ks[0].to(cuda), vs[0].to(cuda), True)
     torch.ops.para_attn.attention_forward_accumulate_(acc, acc_l2, qd, ks[1].to(cuda), vs[1].to(cuda))

@@ -101,7 +101,14 @@ def test_sparse_ranges_with_dense_margins(cuda):
     np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
     with paraattention_amd.StructSparseAttnMode(sparse_mask=bm, sparse_range_query=q_range, sparse_range_key_value=kv_range):
         out2 = torch.nn.functional.scaled_dot_product_attention(q.to(cuda), k.to(cuda), v.to(cuda))
+        # the class-wide switch of the reference's mode (sparse_attn.py:679-692): dense attention while it is off
+        with paraattention_amd.StructSparseAttnMode.disable():
+            assert paraattention_amd.StructSparseAttnMode.disabled
+            dense = torch.nn.functional.scaled_dot_product_attention(q.to(cuda), k.to(cuda), v.to(cuda))
+        assert not paraattention_amd.StructSparseAttnMode.disabled
     assert torch.equal(out, out2)
+    ref_dense, _ = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    np.testing.assert_allclose(dense.float().cpu().numpy(), ref_dense, atol=2e-2, rtol=2e-2)
 
 
 def test_row_without_kept_block(cuda):
