@@ -163,11 +163,52 @@ def test_hunyuan_shape_every_row_by_closed_forms(cuda):
 
 
 def test_wan_cross_attention_shape(cuda):
-    # the Wan 2.1 shape cross-attention: 32760 queries x 512 text keys (reduced heads for the CPU check)
-    q, k, v = inputs.qkv(1, 4, 32760, 512, 128, seed=2)
+    # the Wan 2.1 cross-attention leg at full size: 32760 queries x 40 heads against 512 text keys, every row
+    # against torch's CPU SDPA on identical bits
+    q, k, v = inputs.qkv(1, 40, 32760, 512, 128, seed=2)
     ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q, k, v)
     out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda))
     _check(out, lse, ref_out.float().numpy(), ref_lse.numpy(), "wan-cross")
+
+
+def test_wan_self_attention_shape(cuda):
+    """The Wan 2.1 self-attention leg at full size, B1 H40 S32760 D128 (32760 = 255*128 + 120: a ragged last query
+    tile and a ragged last key tile).  torch's CPU SDPA checks sampled query rows of three heads (first, a middle
+    one, last; the first and last rows of the sequence among them); closed forms that hold at any size check
+    every row of every head: zero keys give LSE = ln(Skv) and out = mean of V, V constant along the keys gives
+    that constant, out is linear in V and LSE does not depend on V."""
+    B, H, S, D = 1, 40, 32760, 128
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=4)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    op = torch.ops.para_attn.attention_forward_with_lse
+    out, lse = op(qd, kd, vd)
+    assert out.shape == (B, H, S, D) and lse.shape == (B, H, S)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    heads = [0, 17, 39]
+    rows = torch.cat([torch.arange(0, 40), torch.arange(S - 130, S), torch.randint(0, S, (86,), generator=torch.Generator().manual_seed(1))])
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, heads][:, :, rows].contiguous(), k[:, heads].contiguous(), v[:, heads].contiguous())
+    got_out, got_lse = out[:, heads][:, :, rows.to(cuda)], lse[:, heads][:, :, rows.to(cuda)]
+    _check(got_out, got_lse, ref_out.float().numpy(), ref_lse.numpy(), "wan-self")
+    # attention_forward is the same launch without the LSE
+    assert torch.equal(torch.ops.para_attn.attention_forward(qd, kd, vd), out)
+    # zero keys
+    out0, lse0 = op(qd, torch.zeros_like(kd), vd)
+    assert (lse0 - np.log(S)).abs().max().item() <= 1e-3
+    assert (out0.float() - vd.float().mean(dim=2, keepdim=True)).abs().max().item() <= 2e-2
+    del out0, lse0
+    # V constant along the keys
+    c = torch.linspace(-2.0, 2.0, D).bfloat16().to(cuda)
+    out_c, lse_c = op(qd, kd, c.expand(B, H, S, D).contiguous())
+    assert (out_c.float() - c.float()).abs().max().item() <= 2e-2
+    assert torch.equal(lse_c, lse)
+    del out_c, lse_c
+    # linearity in V at fixed q, k
+    v2 = torch.roll(vd, 5, dims=2)
+    out2, lse2 = op(qd, kd, v2)
+    out3, lse3 = op(qd, kd, (0.5 * vd.float() - 0.25 * v2.float()).bfloat16())
+    assert torch.equal(lse2, lse) and torch.equal(lse3, lse)
+    err = (out3.float() - (0.5 * out.float() - 0.25 * out2.float())).abs()
+    assert (err <= 2e-2 + 2e-2 * out3.float().abs()).all(), err.max().item()
 
 
 def test_key_mask_and_sparse_kv(cuda):
