@@ -115,6 +115,27 @@ PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void*
                        size_t workspace_bytes, void* stream);
 
 /*
+ * pa_attn_fwd_lse_ws for callers that cannot allocate device memory or bring
+ * a workspace: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference (whose aten
+ * kernels take scratch from torch's allocator).  The workspace is a buffer of
+ * PA_NOALLOC_SCRATCH_BYTES inside the library's device image, one copy per GPU,
+ * held until the process ends; the call allocates and frees nothing.  Same
+ * arguments, kernels and results as pa_attn_fwd_lse_ws with a workspace of
+ * pa_attn_fwd_workspace_bytes() bytes.  A problem whose launch plan needs more
+ * scratch than the buffer holds is refused with PA_ERR_WORKSPACE (it is not run
+ * unsplit behind the caller's back).  Nothing in the buffer has to survive
+ * between calls and nothing has to be cleared; but all calls on one GPU share
+ * it, so calls that overlap on one GPU (two streams, two threads) race.
+ */
+#define PA_NOALLOC_SCRATCH_BYTES (64u << 20)
+PA_API int pa_attn_fwd_lse_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
+                            int dtype, int B, int H, int Sq, int Skv, int D,
+                            const int64_t q_strides[3], const int64_t k_strides[3],
+                            const int64_t v_strides[3], const int64_t out_strides[3],
+                            float scale, const int32_t* kv_len, int is_causal, void* stream);
+
+/*
  * One step of a same-GPU ring sweep in one launch: attention of q against one
  * key/value block, folded into the running pair (acc_out, acc_lse) by the
  * log-sum-exp merge of pa_merge_lse inside the attention kernel's epilogue.

@@ -22,6 +22,8 @@ PA_DTYPE_BF16 = 0
 PA_DTYPE_F16 = 1
 PA_DTYPE_F32 = 2
 
+PA_NOALLOC_SCRATCH_BYTES = 64 << 20
+
 ABI_VERSION = 3
 
 _vp = ctypes.c_void_p
@@ -46,6 +48,10 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _i,
          _vp, _sz, _vp],
+    ),
+    "pa_attn_fwd_lse_noalloc": (
+        _i,
+        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _i, _vp],
     ),
     "pa_attn_fwd_accumulate": (
         _i,

@@ -2237,6 +2237,52 @@ extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int
   return need;
 }
 
+// ---------------------------------------------------------------------------------------------
+// The dense op for callers that cannot allocate (code under HIP graph capture, tight serving loops):
+// the workspace of pa_attn_fwd_lse_ws lives in a file-scope device array instead of coming from the
+// caller.  Every device the library runs on holds its own copy of the array, at its own address,
+// until the process ends; host code must not pass the array's name to a kernel (on the host it is
+// only a stand-in for the symbol), so the device address is looked up once per device with
+// hipGetSymbolAddress and that pointer is what the kernels receive.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[PA_NOALLOC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device, looked up at the first call on that device.
+static int scratch_address(void** out) {
+  static std::atomic<void*> addr[PA_MAX_DEVICES];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= PA_MAX_DEVICES) PA_FAIL(PA_ERR_UNSUPPORTED, "device index %d beyond the %d this library keeps state for", dev, PA_MAX_DEVICES);
+  void* p = addr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) PA_FAIL(PA_ERR_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    addr[dev].store(p, std::memory_order_release);  // benign race: every thread stores the same address
+  }
+  *out = p;
+  return PA_OK;
+}
+
+extern "C" int pa_attn_fwd_lse_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
+                                       int dtype, int B, int H, int Sq, int Skv, int D,
+                                       const int64_t q_strides[3], const int64_t k_strides[3],
+                                       const int64_t v_strides[3], const int64_t out_strides[3],
+                                       float scale, const int32_t* kv_len, int is_causal, void* stream) {
+  // what the same problem would ask of a caller's workspace (0 for sizes that use none)
+  const size_t need = (k_strides && v_strides) ? pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, k_strides, v_strides) : 0;
+  if (need > (size_t)PA_NOALLOC_SCRATCH_BYTES)
+    PA_FAIL(PA_ERR_WORKSPACE, "this problem's launch plan needs %zu bytes of scratch, the static buffer holds %zu: "
+            "call pa_attn_fwd_lse_ws with a workspace of your own", need, (size_t)PA_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = scratch_address(&ws);
+    if (rc) return rc;
+  }
+  return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                        out_strides, scale, kv_len, is_causal, ws, ws ? (size_t)PA_NOALLOC_SCRATCH_BYTES : 0, stream);
+}
+
 extern "C" size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK) {
   if (Hm <= 0 || nQ <= 0 || nK <= 0) return 0;
   const size_t nseg = (size_t)nQ + 2;
