@@ -114,6 +114,39 @@ PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void*
                        float scale, const int32_t* kv_len, int is_causal, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/* kinds of attention mask taken by pa_attn_fwd_masked */
+#define PA_MASK_BOOL 1 /* bytes; 0 = the key is dropped for that query */
+#define PA_MASK_F32 2  /* fp32 bias added to the scaled score */
+#define PA_MASK_ACT 3  /* bias in the activation type (bf16 / f16) */
+
+/*
+ * Dense attention forward with an attention mask: the attn_mask argument of
+ * para_attn.ops.attention_forward_with_lse / attention_forward
+ * (src/para_attn/ops/__init__.py:78-87: attn_bias of the efficient backend,
+ * :215-223: F.scaled_dot_product_attention), boolean or additive, broadcastable
+ * to [B,H,Sq,Skv].  mask_strides = {batch, head, query, key} in elements, 0 on
+ * a broadcast dimension.  A query row that keeps no key yields out = 0 and
+ * lse = -inf.  Not causal (torch refuses a mask together with is_causal).
+ *
+ * A boolean mask that only selects keys (head and query strides 0: the text
+ * padding masks of src/para_attn/ops/__init__.py:248-299) is scanned on the
+ * device; where it keeps a prefix of the keys in every batch element the fast
+ * dense kernels run with the counts as kv_len, otherwise, and for every other
+ * mask, a kernel that reads the mask per score.  The choice is made on the
+ * device: nothing is read back, so the call can be captured in a HIP graph.
+ * workspace: pa_attn_fwd_masked_workspace_bytes() bytes (16-byte aligned, any
+ * contents); null or short is not an error: the per-score kernel runs.
+ */
+PA_API int pa_attn_fwd_masked(const void* q, const void* k, const void* v, void* out, float* lse,
+                       int dtype, int B, int H, int Sq, int Skv, int D,
+                       const int64_t q_strides[3], const int64_t k_strides[3],
+                       const int64_t v_strides[3], const int64_t out_strides[3], float scale,
+                       const void* mask, int mask_kind, const int64_t mask_strides[4],
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+PA_API size_t pa_attn_fwd_masked_workspace_bytes(int B, int H, int Sq, int Skv, int D,
+                                          const int64_t k_strides[3], const int64_t v_strides[3]);
+
 /*
  * pa_attn_fwd_lse_ws for callers that cannot allocate device memory or bring
  * a workspace: code under HIP graph capture, tight serving loops, harnesses
@@ -207,6 +240,22 @@ PA_API size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK);
 PA_API int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int nQ, int nK, int Skv,
                               int kv_lo, int kv_block, int32_t* runs_ws, size_t runs_ws_bytes,
                               void* stream);
+
+/*
+ * pa_attn_fwd_blocksparse for a mask that serves many calls (every layer and
+ * step of a pipeline under the reference's StructSparseAttnMode,
+ * src/para_attn/sparse_attn.py:643-677, uses one mask): `runs` is what
+ * pa_blocksparse_build_runs wrote for the same Hm, nQ, nK, Skv, kv_lo and
+ * kv_block, and is only read here, so the run extraction (about 50 us at a
+ * [24,256,256] mask) is paid once.  Key ranges in `runs` must lie inside
+ * [0, Skv); the kernel trusts them.
+ */
+PA_API int pa_attn_fwd_blocksparse_runs(const void* q, const void* k, const void* v, void* out, float* lse,
+                                 int dtype, int B, int H, int Sq, int Skv, int D,
+                                 const int64_t q_strides[3], const int64_t k_strides[3],
+                                 const int64_t v_strides[3], const int64_t out_strides[3],
+                                 float scale, int Hm, int nQ, int nK, int q_lo, int q_block,
+                                 const int32_t* runs, size_t runs_bytes, void* stream);
 
 /*
  * One step of the ring-attention partial-result merge, fused into one pass:

@@ -24,6 +24,10 @@ PA_DTYPE_F32 = 2
 
 PA_NOALLOC_SCRATCH_BYTES = 64 << 20
 
+PA_MASK_BOOL = 1
+PA_MASK_F32 = 2
+PA_MASK_ACT = 3
+
 ABI_VERSION = 3
 
 _vp = ctypes.c_void_p
@@ -49,6 +53,12 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _i,
          _vp, _sz, _vp],
     ),
+    "pa_attn_fwd_masked": (
+        _i,
+        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f,
+         _vp, _i, _strides, _vp, _sz, _vp],
+    ),
+    "pa_attn_fwd_masked_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _strides, _strides]),
     "pa_attn_fwd_lse_noalloc": (
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _i, _vp],
@@ -63,6 +73,11 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f,
          _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp],
+    ),
+    "pa_attn_fwd_blocksparse_runs": (
+        _i,
+        [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f,
+         _i, _i, _i, _i, _i, _vp, _sz, _vp],
     ),
     "pa_blocksparse_workspace_bytes": (_sz, [_i, _i, _i]),
     "pa_blocksparse_build_runs": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),

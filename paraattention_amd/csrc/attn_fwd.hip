@@ -86,7 +86,18 @@ struct AttnParams {
   float* acc_out;
   float* acc_lse;
   int acc_first;
+  // attn_fwd_kernel only: an attention mask, one element per (batch, head, query, key) reached through four
+  // strides in elements (0 on broadcast dimensions).  MASK_BOOL: bytes, 0 = the key is dropped for that query;
+  // MASK_F32 / MASK_ACT: a bias added to the scaled score (fp32, or the activation type).
+  const void* mask;
+  int64_t ms_b, ms_h, ms_q, ms_k;
+  // dense kernels: with `gate` set the launch leaves at once unless *gate == gate_want (a decision taken on
+  // the device by an earlier launch of the same stream, e.g. whether a key mask is a prefix)
+  const int* gate;
+  int gate_want;
 };
+
+constexpr int MASK_NONE = 0, MASK_BOOL = 1, MASK_F32 = 2, MASK_ACT = 3;
 
 template <int D>
 struct Smem {
@@ -198,10 +209,13 @@ __device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int he
 
 }
 
-template <typename T, int D, bool SPARSE>
+template <typename T, int D, bool SPARSE, int MASK = MASK_NONE>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
   typedef Smem<D> SM;
+  if constexpr (!SPARSE) {
+    if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  }
   constexpr int DC = D / 16;   // contraction chunks of the first GEMM
   constexpr int DB = D / 32;   // 32-row blocks of O^T
   constexpr int CH = D / 8;    // 16-byte chunks per K/V row
@@ -386,6 +400,29 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
       }
     }
 
+    // ---- attention mask: this lane's query row against the tile's keys ------------
+    if constexpr (MASK != MASK_NONE) {
+      const int64_t mrow = (int64_t)batch * p.ms_b + (int64_t)head * p.ms_h + (int64_t)(row_ok ? my_row : row_end - 1) * p.ms_q;
+      const float per_scale = 1.0f / (c * LN2);  // bias / scale, so that (s + that) * c = s * c + bias * log2(e)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
+          if (n < cur_valid) {  // keys past the end are dealt with below and must not be read
+            const int64_t mi = mrow + (int64_t)(cur_n0 + n) * p.ms_k;
+            if constexpr (MASK == MASK_BOOL) {
+              if (((const uint8_t*)p.mask)[mi] == 0) s[t][r] = -INFINITY;
+            } else if constexpr (MASK == MASK_F32) {
+              s[t][r] += ((const float*)p.mask)[mi] * per_scale;
+            } else {
+              const uint32_t w = ((const uint16_t*)p.mask)[mi];
+              s[t][r] += T::lo(w) * per_scale;
+            }
+          }
+        }
+    }
+
     // ---- mask the ragged end of a range ---------------------------------------
     if (cur_valid < BN || (!SPARSE && p.causal && cur_n0 + BN - 1 > wave_row0)) {
       int lim = cur_valid;
@@ -409,7 +446,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const float mx_s = mx * c;
     if (__any(mx_s > m_run + RESCALE_SLACK)) {
       const float m_new = fmaxf(m_run, mx_s);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      // the branch is taken by the whole wavefront: a row that has seen no kept key yet (possible under a mask
+      // only) still has no maximum, and -inf - -inf must not turn its zeros into NaN
+      if (MASK != MASK_NONE && m_new == -INFINITY) alpha = 1.f;
       l_run *= alpha;
 #pragma unroll
       for (int i = 0; i < DB; ++i)
@@ -419,12 +459,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     }
     uint32_t pk[2][8];
     float lsum = 0.f;
+    // a row whose keys so far were all masked away has no maximum yet: exponentiate against 0 (every term is 0)
+    const float m_use = (MASK != MASK_NONE && m_run == -INFINITY) ? 0.f : m_run;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], c, -m_run));
-        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], c, -m_run));
+        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], c, -m_use));
+        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], c, -m_use));
         lsum += p0 + p1;
         pk[t][r >> 1] = T::pack2(p0, p1);
       }
@@ -502,6 +544,9 @@ template <typename T, bool SPARSE>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
   constexpr int D = 128, DC = 8, DB = 4;
+  if constexpr (!SPARSE) {
+    if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  }
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                    // [2][64][256 B]
   char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
@@ -844,6 +889,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   // the reference point of the softmax stays 0 and row maxima, rescale checks and rescales are compiled out.
   if constexpr (!SPARSE && NW == 8) {
     if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
+  }
+  if constexpr (!SPARSE) {
+    if (p.gate != nullptr && *p.gate != p.gate_want) return;
   }
   constexpr int RS = 4 * NW;    // tile rows between two of them
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
@@ -1302,6 +1350,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
   // BOUNDED and the flag: as in attn_fwd_d128_pipe_kernel
   if constexpr (!SPARSE) {
     if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
+    if (p.gate != nullptr && *p.gate != p.gate_want) return;
   }
   typedef typename T::vec8 vec8;
   constexpr int DC = 4, DB = 2;
@@ -1627,6 +1676,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
 // once.  One thread = 8 consecutive output elements of one query row; 16 rows per workgroup.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_split_merge_kernel(const AttnParams p) {
+  if (p.gate != nullptr && *p.gate != p.gate_want) return;
   const int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int c8 = (threadIdx.x & 15) * 8;
   const int tl = (int)(r / p.bm), local = (int)(r % p.bm);
@@ -1840,6 +1890,40 @@ __global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part
   }
 }
 
+// A key-only boolean mask [B, Skv] (byte strides mb, mk): per batch element the number of kept keys, and
+// whether in every batch element the kept keys are exactly the leading ones (then the dense kernels take the
+// counts as kv_len and the mask need not be looked at again).  One workgroup; out[0..B) = counts,
+// out[B] = 1 if all are prefixes else 0.
+__global__ __launch_bounds__(1024) void key_mask_scan_kernel(const uint8_t* mask, int64_t mb, int64_t mk, int B,
+                                                             int Skv, int32_t* out) {
+  __shared__ int s_cnt[1024];
+  __shared__ int s_last[1024];
+  int all_prefix = 1;
+  for (int b = 0; b < B; ++b) {
+    int cnt = 0, last = -1;
+    for (int j = threadIdx.x; j < Skv; j += 1024) {
+      if (mask[(int64_t)b * mb + (int64_t)j * mk] != 0) {
+        ++cnt;
+        last = j;
+      }
+    }
+    s_cnt[threadIdx.x] = cnt;
+    s_last[threadIdx.x] = last;
+    __syncthreads();
+    for (int d = 512; d > 0; d >>= 1) {
+      if ((int)threadIdx.x < d) {
+        s_cnt[threadIdx.x] += s_cnt[threadIdx.x + d];
+        s_last[threadIdx.x] = max(s_last[threadIdx.x], s_last[threadIdx.x + d]);
+      }
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) out[b] = s_cnt[0];
+    if (s_cnt[0] != s_last[0] + 1) all_prefix = 0;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[B] = all_prefix;
+}
+
 }  // namespace pa
 
 using namespace pa;
@@ -1889,6 +1973,8 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.acc_out = nullptr; p.acc_lse = nullptr; p.acc_first = 0;
   p.split_main = 0; p.split_tiles = 0; p.split_s = 0; p.ws_out = nullptr; p.ws_lse = nullptr;
   p.bound_flag = nullptr;
+  p.mask = nullptr; p.ms_b = p.ms_h = p.ms_q = p.ms_k = 0;
+  p.gate = nullptr; p.gate_want = 0;
 }
 
 template <typename T, int D, bool SPARSE>
@@ -2140,7 +2226,8 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
                           const int64_t q_strides[3], const int64_t k_strides[3],
                           const int64_t v_strides[3], const int64_t out_strides[3], float scale,
                           const int32_t* kv_len, int is_causal, void* workspace, size_t workspace_bytes,
-                          void* stream, float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0) {
+                          void* stream, float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0,
+                          const int* gate = nullptr, int gate_want = 0) {
   const int64_t zero3[3] = {0, 0, 0};
   const bool accumulate = acc_out != nullptr;
   if (accumulate) {
@@ -2156,6 +2243,8 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
   p.kv_len = kv_len;
   p.causal = is_causal != 0;
+  p.gate = gate;
+  p.gate_want = gate_want;
   // a workspace that has room for them beside the key split's partials starts with BOUND_WS_BYTES for the score bound
   const size_t ws_avail = workspace ? workspace_bytes : 0;
   char* ws_base = (char*)workspace;
@@ -2237,6 +2326,89 @@ extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int
   return need;
 }
 
+// The generic kernel with an attention mask (any head_dim it is built for, any strides).
+template <typename T, int D>
+static int launch_masked(const AttnParams& p, int mask_kind, hipStream_t stream) {
+  const int64_t nblocks = (int64_t)p.B * p.H * p.n_qtiles;
+  if (nblocks == 0) return PA_OK;
+  const void* fn = mask_kind == MASK_BOOL ? (const void*)attn_fwd_kernel<T, D, false, MASK_BOOL>
+                   : mask_kind == MASK_F32 ? (const void*)attn_fwd_kernel<T, D, false, MASK_F32>
+                                           : (const void*)attn_fwd_kernel<T, D, false, MASK_ACT>;
+  const size_t smem = Smem<D>::BYTES;
+  static bool attr_done[PA_MAX_DEVICES][4] = {};  // benign race: the call is idempotent
+  const int dev = current_device();
+  if (dev < 0 || !attr_done[dev][mask_kind]) {
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    if (dev >= 0) attr_done[dev][mask_kind] = true;
+  }
+  if (mask_kind == MASK_BOOL)
+    hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, MASK_BOOL>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+  else if (mask_kind == MASK_F32)
+    hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, MASK_F32>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+  else
+    hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, MASK_ACT>), dim3((unsigned)nblocks), dim3(NTHREADS), smem, stream, p);
+  PA_CHECK_LAUNCH("masked attention kernel");
+  return PA_OK;
+}
+
+// Words at the front of pa_attn_fwd_masked's workspace: kept-key counts per batch element and the prefix flag.
+static size_t mask_scan_bytes(int B) { return (((size_t)B + 1) * sizeof(int32_t) + 255) & ~(size_t)255; }
+
+extern "C" size_t pa_attn_fwd_masked_workspace_bytes(int B, int H, int Sq, int Skv, int D,
+                                                     const int64_t k_strides[3], const int64_t v_strides[3]) {
+  if (B <= 0) return 0;
+  return mask_scan_bytes(B) + pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, k_strides, v_strides);
+}
+
+extern "C" int pa_attn_fwd_masked(const void* q, const void* k, const void* v, void* out, float* lse,
+                                  int dtype, int B, int H, int Sq, int Skv, int D,
+                                  const int64_t q_strides[3], const int64_t k_strides[3],
+                                  const int64_t v_strides[3], const int64_t out_strides[3], float scale,
+                                  const void* mask, int mask_kind, const int64_t mask_strides[4],
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides, scale);
+  if (rc) return rc;
+  if (mask_kind != MASK_BOOL && mask_kind != MASK_F32 && mask_kind != MASK_ACT)
+    PA_FAIL(PA_ERR_INVALID, "mask kind %d is none of PA_MASK_BOOL, PA_MASK_F32, PA_MASK_ACT", mask_kind);
+  if (!mask_strides) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  const bool any = B > 0 && H > 0 && Sq > 0 && Skv > 0;
+  if (any && !mask) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  for (int i = 0; i < 4; ++i)
+    if (mask_strides[i] < 0) PA_FAIL(PA_ERR_UNSUPPORTED, "mask has a negative stride");
+  if (workspace && ((uintptr_t)workspace) % 16) PA_FAIL(PA_ERR_WORKSPACE, "attention workspace not 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  AttnParams p;
+  fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
+  p.bm = BM;
+  p.n_qtiles = (Sq + BM - 1) / BM;
+  p.mask = mask;
+  p.ms_b = mask_strides[0]; p.ms_h = mask_strides[1]; p.ms_q = mask_strides[2]; p.ms_k = mask_strides[3];
+  // A boolean mask that only selects keys (the same for every head and query row; what the text padding of
+  // video DiTs looks like) is usually a prefix per batch element.  Whether it is, is found out on the device: a
+  // small scan writes the kept-key counts and a flag, then both the dense launch (counts as kv_len) and the
+  // masked launch are enqueued, and the one the flag does not select leaves at once.  Nothing is read back.
+  const bool key_only = mask_kind == MASK_BOOL && (H == 1 || p.ms_h == 0) && (Sq == 1 || p.ms_q == 0);
+  const size_t scan = mask_scan_bytes(B);
+  if (key_only && any && workspace && workspace_bytes >= scan) {
+    int32_t* words = (int32_t*)workspace;
+    hipLaunchKernelGGL(key_mask_scan_kernel, dim3(1), dim3(1024), 0, st, (const uint8_t*)mask, p.ms_b, p.ms_k, B, Skv, words);
+    PA_CHECK_LAUNCH("key mask scan kernel");
+    rc = attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
+                        scale, words, 0, (char*)workspace + scan, workspace_bytes - scan, stream, nullptr, nullptr, 0,
+                        words + B, 1);
+    if (rc) return rc;
+    p.gate = words + B;
+    p.gate_want = 0;
+  }
+  if (!any) {  // no rows, or no keys: the dense path writes what an empty softmax gives
+    return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
+                          scale, nullptr, 0, nullptr, 0, stream);
+  }
+  if (dtype == PA_DTYPE_BF16) return D == 128 ? launch_masked<BF16, 128>(p, mask_kind, st) : launch_masked<BF16, 64>(p, mask_kind, st);
+  return D == 128 ? launch_masked<F16, 128>(p, mask_kind, st) : launch_masked<F16, 64>(p, mask_kind, st);
+}
+
 // ---------------------------------------------------------------------------------------------
 // The dense op for callers that cannot allocate (code under HIP graph capture, tight serving loops):
 // the workspace of pa_attn_fwd_lse_ws lives in a file-scope device array instead of coming from the
@@ -2308,24 +2480,15 @@ extern "C" int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int 
   return PA_OK;
 }
 
-extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void* v, void* out,
-                                       float* lse, int dtype, int B, int H, int Sq, int Skv, int D,
-                                       const int64_t q_strides[3], const int64_t k_strides[3],
-                                       const int64_t v_strides[3], const int64_t out_strides[3],
-                                       float scale, const uint8_t* block_mask, int Hm, int nQ, int nK,
-                                       int q_lo, int q_block, int kv_lo, int kv_block,
-                                       int32_t* runs_ws, size_t runs_ws_bytes, void* stream) {
-  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
-                        out_strides, scale);
-  if (rc) return rc;
-  if (Hm != 1 && Hm != H) PA_FAIL(PA_ERR_INVALID, "block mask heads must be 1 or H=%d (got %d)", H, Hm);
-  if (q_block <= 0 || q_lo < 0 || (int64_t)q_lo + (int64_t)nQ * q_block > Sq)
-    PA_FAIL(PA_ERR_INVALID, "query blocks [%d + %d*%d) exceed Sq=%d", q_lo, nQ, q_block, Sq);
-  rc = pa_blocksparse_build_runs(block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, runs_ws, runs_ws_bytes, stream);
-  if (rc) return rc;
+// Shared tail of the two block-sparse entry points: `runs` already holds the key ranges.
+static int blocksparse_launch(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                              int B, int H, int Sq, int Skv, int D, const int64_t q_strides[3],
+                              const int64_t k_strides[3], const int64_t v_strides[3],
+                              const int64_t out_strides[3], float scale, int Hm, int nQ, int nK, int q_lo,
+                              int q_block, const int32_t* runs, void* stream) {
   AttnParams p;
   fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
-  p.runs = runs_ws;
+  p.runs = runs;
   p.Hm = Hm; p.nQ = nQ; p.cap = nK / 2 + 3;
   p.q_lo = q_lo; p.q_block = q_block;
   choose_kernel(p, D, (q_block % 256 == 0 && q_lo % 256 == 0) ? 256 : 128, false, 0, nullptr);
@@ -2337,4 +2500,47 @@ extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void*
   if (D == 128 && p.pipe && !tuning().no_xcd_order)
     p.xcd_chunk = (int)(((int64_t)B * H * p.n_qtiles + 7) / 8);
   return dispatch_attn<true>(p, dtype, D, (hipStream_t)stream);
+}
+
+static int blocksparse_check(const void* q, const void* k, const void* v, void* out, int dtype, int B, int H,
+                             int Sq, int Skv, int D, const int64_t* qs, const int64_t* ks, const int64_t* vs,
+                             const int64_t* os, float scale, int Hm, int nQ, int nK, int q_lo, int q_block) {
+  int rc = check_common(q, k, v, out, dtype, B, H, Sq, Skv, D, qs, ks, vs, os, scale);
+  if (rc) return rc;
+  if (Hm != 1 && Hm != H) PA_FAIL(PA_ERR_INVALID, "block mask heads must be 1 or H=%d (got %d)", H, Hm);
+  if (nQ <= 0 || nK <= 0) PA_FAIL(PA_ERR_INVALID, "bad block mask geometry");
+  if (q_block <= 0 || q_lo < 0 || (int64_t)q_lo + (int64_t)nQ * q_block > Sq)
+    PA_FAIL(PA_ERR_INVALID, "query blocks [%d + %d*%d) exceed Sq=%d", q_lo, nQ, q_block, Sq);
+  return PA_OK;
+}
+
+extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void* v, void* out,
+                                       float* lse, int dtype, int B, int H, int Sq, int Skv, int D,
+                                       const int64_t q_strides[3], const int64_t k_strides[3],
+                                       const int64_t v_strides[3], const int64_t out_strides[3],
+                                       float scale, const uint8_t* block_mask, int Hm, int nQ, int nK,
+                                       int q_lo, int q_block, int kv_lo, int kv_block,
+                                       int32_t* runs_ws, size_t runs_ws_bytes, void* stream) {
+  int rc = blocksparse_check(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
+                             scale, Hm, nQ, nK, q_lo, q_block);
+  if (rc) return rc;
+  rc = pa_blocksparse_build_runs(block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, runs_ws, runs_ws_bytes, stream);
+  if (rc) return rc;
+  return blocksparse_launch(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                            out_strides, scale, Hm, nQ, nK, q_lo, q_block, runs_ws, stream);
+}
+
+extern "C" int pa_attn_fwd_blocksparse_runs(const void* q, const void* k, const void* v, void* out,
+                                            float* lse, int dtype, int B, int H, int Sq, int Skv, int D,
+                                            const int64_t q_strides[3], const int64_t k_strides[3],
+                                            const int64_t v_strides[3], const int64_t out_strides[3],
+                                            float scale, int Hm, int nQ, int nK, int q_lo, int q_block,
+                                            const int32_t* runs, size_t runs_bytes, void* stream) {
+  int rc = blocksparse_check(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
+                             scale, Hm, nQ, nK, q_lo, q_block);
+  if (rc) return rc;
+  if (!runs) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  if (runs_bytes < pa_blocksparse_workspace_bytes(Hm, nQ, nK)) PA_FAIL(PA_ERR_WORKSPACE, "runs buffer too small for this mask geometry");
+  return blocksparse_launch(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                            out_strides, scale, Hm, nQ, nK, q_lo, q_block, runs, stream);
 }

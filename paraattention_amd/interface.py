@@ -41,8 +41,14 @@ def kernel_takes(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=Fal
     if query.requires_grad or key.requires_grad or value.requires_grad:
         return False  # forward only, like the reference's ops (src/para_attn/ops/__init__.py:203-211)
     if attn_mask is not None:
-        # a boolean mask over keys only, the same for every query row
-        if attn_mask.dtype != torch.bool or attn_mask.ndim != 4 or attn_mask.shape[-2] != 1 or attn_mask.shape[1] != 1:
+        # boolean or additive, broadcastable to the scores as torch's SDPA reads it (trailing dimensions aligned)
+        if not isinstance(attn_mask, torch.Tensor) or attn_mask.ndim > 4 or attn_mask.device != query.device:
+            return False
+        if attn_mask.dtype != torch.bool and not attn_mask.is_floating_point():
+            return False
+        full = (query.shape[0], query.shape[1], query.shape[2], key.shape[2])
+        shape = (1,) * (4 - attn_mask.ndim) + tuple(attn_mask.shape)
+        if any(s not in (1, f) for s, f in zip(shape, full)):
             return False
     return True
 

@@ -17,6 +17,7 @@ torch elementwise calls:
   merge_attention_lse / merge_attention_lse_   (torch _SDPAMerger._merge_one)
   attention_forward_accumulate_ / _final       (attention + merge step in one launch)
   attention_forward_block_sparse               (sparse_attn.py:74-278)
+  block_sparse_key_runs, attention_forward_block_sparse_runs  (the same with the mask's run scan done once)
   fbcache_residual_diff                        (first_block_cache/utils.py:228-233)
   fbcache_first_residual_diff, fbcache_apply_residual (utils.py:359, 237-259)
   taylorseer_derivatives, taylorseer_value     (first_block_cache/taylorseer.py:29-48)
@@ -65,26 +66,6 @@ def _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask=None, ca
         raise ValueError(f"key shape {tuple(key.shape)} does not match query {tuple(query.shape)}")
     if value.shape[:3] != key.shape[:3] or value.shape[3] != D:
         raise ValueError(f"value shape {tuple(value.shape)} does not match key {tuple(key.shape)}")
-
-
-def _key_keep_vector(attn_mask, B, Skv):
-    """Reduce a boolean mask that only selects keys to [B, Skv], or return None.
-
-    Accepts the shapes the reference's sparse_kv op accepts (any leading dims,
-    reduced to their first head / first query row, src/para_attn/ops/__init__.py:280-282).
-    """
-    m = attn_mask
-    if m.dtype != torch.bool or m.shape[-1] != Skv:
-        return None
-    while m.ndim > 2:
-        if m.shape[1] != 1:
-            return None
-        m = m[:, 0]
-    if m.ndim == 1:
-        m = m.unsqueeze(0)
-    if m.shape[0] not in (1, B):
-        return None
-    return m.expand(B, Skv)
 
 
 def _dense_forward(query, key, value, scale, want_lse, kv_len=None, is_causal=False):
@@ -143,26 +124,61 @@ def _accumulate_forward(acc_out, acc_lse, query, key, value, scale, first, final
     return out
 
 
+def _broadcast_mask(attn_mask, B, H, Sq, Skv, dtype):
+    """The mask as torch's SDPA reads it: trailing dimensions aligned with [B,H,Sq,Skv], every dimension full or 1
+    (src/para_attn/ops/__init__.py:215-223 hands it to F.scaled_dot_product_attention as it came).  Returns
+    (tensor to pass, mask kind, (batch, head, query, key) strides in elements with 0 on broadcast dimensions)."""
+    m = attn_mask
+    if m.ndim > 4:
+        raise ValueError(f"attn_mask has {m.ndim} dimensions; at most 4 ([B,H,Sq,Skv]) broadcast against the scores")
+    while m.ndim < 4:
+        m = m.unsqueeze(0)
+    full = (B, H, Sq, Skv)
+    for d in range(4):
+        if m.shape[d] not in (1, full[d]):
+            raise ValueError(f"attn_mask shape {tuple(attn_mask.shape)} does not broadcast to {full}")
+    if m.dtype == torch.bool:
+        kind = _lib.PA_MASK_BOOL
+    elif m.dtype == torch.float32:
+        kind = _lib.PA_MASK_F32
+    elif m.dtype == dtype:
+        kind = _lib.PA_MASK_ACT
+    elif m.is_floating_point():
+        m, kind = m.float(), _lib.PA_MASK_F32
+    else:
+        raise ValueError(f"attn_mask must be boolean or floating point, got {m.dtype}")
+    strides = [0 if m.shape[d] == 1 else m.stride(d) for d in range(4)]
+    return m, kind, (ctypes.c_int64 * 4)(*strides)
+
+
 def _masked_forward(query, key, value, attn_mask, scale, want_lse, is_causal=False):
-    """attn_mask / is_causal handling shared by the three SDPA-signature ops."""
+    """attn_mask / is_causal handling shared by the three SDPA-signature ops.  Nothing here reads the mask on
+    the host: whether a key mask is a prefix is settled on the device (pa_attn_fwd_masked), so masked calls can
+    be captured in a HIP graph like the unmasked ones."""
     if attn_mask is None:
         return _dense_forward(query, key, value, scale, want_lse, is_causal=is_causal)
-    B, Skv = query.shape[0], key.shape[2]
-    keep = _key_keep_vector(attn_mask, B, Skv)
-    if keep is None:
-        raise NotImplementedError(
-            "attn_mask must be None or a boolean mask over keys only ([B,1,1,Skv]-like); "
-            "per-query masks go through attention_forward_block_sparse"
+    B, H, Sq, D = query.shape
+    Skv = key.shape[2]
+    mask, kind, mstrides = _broadcast_mask(attn_mask, B, H, Sq, Skv, query.dtype)
+    q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
+    out = torch.empty_like(q)
+    if out.stride(-1) != 1:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        ks, vs = _lib.strides3(k), _lib.strides3(v)
+        ws_bytes = lib.pa_attn_fwd_masked_workspace_bytes(B, H, Sq, Skv, D, ks, vs)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+        rc = lib.pa_attn_fwd_masked(
+            _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
+            _lib.strides3(q), ks, vs, _lib.strides3(out), float(scale),
+            _ptr(mask), kind, mstrides, _ptr(ws), ws_bytes, _stream_ptr(q.device),
         )
-    lens = keep.sum(-1, dtype=torch.int32)
-    prefix = torch.arange(Skv, device=keep.device).unsqueeze(0) < lens.unsqueeze(1)
-    if not bool((keep == prefix).all()):
-        # kept keys are scattered: move them to the front (stable), then treat as a prefix
-        order = torch.argsort((~keep).to(torch.uint8), dim=-1, stable=True)
-        idx = order[:, None, :, None].expand(B, key.shape[1], Skv, key.shape[3])
-        key = torch.gather(key, 2, idx)
-        value = torch.gather(value, 2, idx)
-    return _dense_forward(query, key, value, scale, want_lse, kv_len=lens.contiguous())
+    _lib.check(rc, "pa_attn_fwd_masked")
+    return out, lse
 
 
 # ---------------------------------------------------------------------------------
@@ -241,6 +257,8 @@ def attention_forward_sparse_kv(
     if attn_mask.dtype != torch.bool:
         raise AssertionError("attn_mask must be a boolean tensor")
     m = attn_mask
+    if m.shape[-1] != key.shape[2]:
+        raise ValueError(f"attn_mask's last dimension {m.shape[-1]} is not the key length {key.shape[2]}")
     if m.shape[0] != query.shape[0]:
         m = m.expand(query.shape[0], *m.shape[1:])
     while m.ndim > 2:
@@ -386,6 +404,38 @@ def _(acc_out, acc_lse, query, key, value, *, scale=None):
 # ---------------------------------------------------------------------------------
 # block-sparse attention
 # ---------------------------------------------------------------------------------
+def _sparse_geometry(query, key, block_mask_shape, q_lo, q_hi, kv_lo, kv_hi):
+    """Checks the block-mask geometry against the tensors (src/para_attn/sparse_attn.py:112-131) and returns
+    (Hm, nQ, nK, q_lo, q_hi, kv_lo, kv_hi, q_block, kv_block)."""
+    B, H, Sq, D = query.shape
+    Skv = key.shape[2]
+    q_hi = Sq if q_hi < 0 else q_hi
+    kv_hi = Skv if kv_hi < 0 else kv_hi
+    if len(block_mask_shape) != 3 or block_mask_shape[0] not in (1, H):
+        raise ValueError(f"block_mask must be [nQ,nK] or [H,nQ,nK], got {tuple(block_mask_shape)}")
+    Hm, nQ, nK = block_mask_shape
+    if not (0 <= q_lo <= q_hi <= Sq):
+        raise ValueError(f"sparse query range must be in [0, {Sq}], got {(q_lo, q_hi)}")
+    if not (0 <= kv_lo <= kv_hi <= Skv):
+        raise ValueError(f"sparse key/value range must be in [0, {Skv}], got {(kv_lo, kv_hi)}")
+    if nQ == 0 or nK == 0 or (q_hi - q_lo) % nQ or (kv_hi - kv_lo) % nK:
+        raise ValueError("block_mask must divide the sparse query and key/value ranges")
+    q_block = (q_hi - q_lo) // nQ
+    kv_block = (kv_hi - kv_lo) // nK
+    if q_block == 0 or kv_block == 0:
+        raise ValueError("empty sparse range")
+    return Hm, nQ, nK, q_lo, q_hi, kv_lo, kv_hi, q_block, kv_block
+
+
+def _sparse_outputs(query):
+    q = _kernel_ready(query)
+    out = torch.empty_like(q)
+    if out.stride(-1) != 1:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    B, H, Sq, _ = q.shape
+    return q, out, torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+
+
 @torch.library.custom_op("para_attn::attention_forward_block_sparse", mutates_args=(), device_types=("cuda",))
 def attention_forward_block_sparse(
     query: torch.Tensor,
@@ -411,30 +461,13 @@ def attention_forward_block_sparse(
     _check_sdpa_args(query, key, value, 0.0, False)
     B, H, Sq, D = query.shape
     Skv = key.shape[2]
-    q_hi = Sq if q_hi < 0 else q_hi
-    kv_hi = Skv if kv_hi < 0 else kv_hi
     if block_mask.dtype != torch.bool:
         raise ValueError("block_mask must be boolean")
     if block_mask.ndim == 2:
         block_mask = block_mask.unsqueeze(0)
-    if block_mask.ndim != 3 or block_mask.shape[0] not in (1, H):
-        raise ValueError(f"block_mask must be [nQ,nK] or [H,nQ,nK], got {tuple(block_mask.shape)}")
-    Hm, nQ, nK = block_mask.shape
-    if not (0 <= q_lo <= q_hi <= Sq):
-        raise ValueError(f"sparse query range must be in [0, {Sq}], got {(q_lo, q_hi)}")
-    if not (0 <= kv_lo <= kv_hi <= Skv):
-        raise ValueError(f"sparse key/value range must be in [0, {Skv}], got {(kv_lo, kv_hi)}")
-    if nQ == 0 or nK == 0 or (q_hi - q_lo) % nQ or (kv_hi - kv_lo) % nK:
-        raise ValueError("block_mask must divide the sparse query and key/value ranges")
-    q_block = (q_hi - q_lo) // nQ
-    kv_block = (kv_hi - kv_lo) // nK
-    if q_block == 0 or kv_block == 0:
-        raise ValueError("empty sparse range")
-    q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
-    out = torch.empty_like(q)
-    if out.stride(-1) != 1:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    Hm, nQ, nK, q_lo, q_hi, kv_lo, kv_hi, q_block, kv_block = _sparse_geometry(query, key, block_mask.shape, q_lo, q_hi, kv_lo, kv_hi)
+    k, v = _kernel_ready(key), _kernel_ready(value)
+    q, out, lse = _sparse_outputs(query)
     mask_u8 = block_mask.contiguous().view(torch.uint8)
     lib = _lib.load()
     ws_bytes = lib.pa_blocksparse_workspace_bytes(Hm, nQ, nK)
@@ -458,6 +491,88 @@ def _(query, key, value, block_mask, q_lo=0, q_hi=-1, kv_lo=0, kv_hi=-1, *, scal
     return query.new_empty((B, H, Sq, value.shape[-1])), query.new_empty((B, H, Sq), dtype=torch.float32)
 
 
+@torch.library.custom_op("para_attn::block_sparse_key_runs", mutates_args=(), device_types=("cuda",))
+def block_sparse_key_runs(block_mask: torch.Tensor, seq_kv: int, kv_lo: int = 0, kv_hi: int = -1) -> torch.Tensor:
+    """The key ranges of a block mask, as the block-sparse kernel walks them: the mask's runs of kept blocks per
+    (mask head, query block), merged with the dense key margins (the scan of src/para_attn/sparse_attn.py:215-234).
+    Returns the int32 buffer ``attention_forward_block_sparse_runs`` takes; build it once for a mask that serves
+    many calls.  ``block_sparse_runs`` gives a structured view of it."""
+    if block_mask.dtype != torch.bool:
+        raise ValueError("block_mask must be boolean")
+    if block_mask.ndim == 2:
+        block_mask = block_mask.unsqueeze(0)
+    if block_mask.ndim != 3 or 0 in block_mask.shape:
+        raise ValueError(f"block_mask must be [nQ,nK] or [H,nQ,nK], got {tuple(block_mask.shape)}")
+    Hm, nQ, nK = block_mask.shape
+    kv_hi = seq_kv if kv_hi < 0 else kv_hi
+    if not (0 <= kv_lo <= kv_hi <= seq_kv) or (kv_hi - kv_lo) % nK or kv_hi == kv_lo:
+        raise ValueError("block_mask must divide a non-empty sparse key/value range inside the keys")
+    kv_block = (kv_hi - kv_lo) // nK
+    lib = _lib.load()
+    ws_bytes = lib.pa_blocksparse_workspace_bytes(Hm, nQ, nK)
+    ws = torch.zeros((ws_bytes + 3) // 4, dtype=torch.int32, device=block_mask.device)
+    mask_u8 = block_mask.contiguous().view(torch.uint8)
+    with torch.cuda.device(block_mask.device):
+        rc = lib.pa_blocksparse_build_runs(
+            _ptr(mask_u8), Hm, nQ, nK, seq_kv, kv_lo, kv_block, _ptr(ws), ws_bytes, _stream_ptr(block_mask.device)
+        )
+    _lib.check(rc, "pa_blocksparse_build_runs")
+    return ws
+
+
+@torch.library.register_fake("para_attn::block_sparse_key_runs")
+def _(block_mask, seq_kv, kv_lo=0, kv_hi=-1):
+    Hm, nQ, nK = block_mask.shape if block_mask.ndim == 3 else (1, *block_mask.shape)
+    nseg, cap = nQ + 2, nK // 2 + 3
+    return block_mask.new_empty((Hm * nseg + Hm * nseg * cap * 2,), dtype=torch.int32)
+
+
+@torch.library.custom_op("para_attn::attention_forward_block_sparse_runs", mutates_args=(), device_types=("cuda",))
+def attention_forward_block_sparse_runs(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    runs: torch.Tensor,
+    mask_heads: int,
+    n_q: int,
+    n_k: int,
+    q_lo: int = 0,
+    q_hi: int = -1,
+    *,
+    scale: Optional[float] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``attention_forward_block_sparse`` with the key ranges already extracted: ``runs`` is the result of
+    ``block_sparse_key_runs`` for a [mask_heads, n_q, n_k] mask over keys of the same length (and the same
+    sparse key range).  Saves the extraction on every call after the first."""
+    _check_sdpa_args(query, key, value, 0.0, False)
+    B, H, Sq, D = query.shape
+    Skv = key.shape[2]
+    if runs.dtype != torch.int32 or not runs.is_contiguous() or runs.device != query.device:
+        raise ValueError("runs must be the contiguous int32 tensor block_sparse_key_runs returned, on the query's device")
+    Hm, nQ, nK, q_lo, q_hi, _, _, q_block, _ = _sparse_geometry(query, key, (mask_heads, n_q, n_k), q_lo, q_hi, 0, n_k)
+    lib = _lib.load()
+    if runs.numel() * 4 < lib.pa_blocksparse_workspace_bytes(Hm, nQ, nK):
+        raise ValueError(f"runs holds {runs.numel()} words, too few for a [{Hm},{nQ},{nK}] mask: not the result of block_sparse_key_runs for it")
+    k, v = _kernel_ready(key), _kernel_ready(value)
+    q, out, lse = _sparse_outputs(query)
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    with torch.cuda.device(q.device):
+        rc = lib.pa_attn_fwd_blocksparse_runs(
+            _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,
+            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out), float(scale),
+            Hm, nQ, nK, q_lo, q_block, _ptr(runs), runs.numel() * 4, _stream_ptr(q.device),
+        )
+    _lib.check(rc, "pa_attn_fwd_blocksparse_runs")
+    return out, lse
+
+
+@torch.library.register_fake("para_attn::attention_forward_block_sparse_runs")
+def _(query, key, value, runs, mask_heads, n_q, n_k, q_lo=0, q_hi=-1, *, scale=None):
+    B, H, Sq, _ = query.shape
+    return query.new_empty((B, H, Sq, value.shape[-1])), query.new_empty((B, H, Sq), dtype=torch.float32)
+
+
 def block_sparse_runs(block_mask, Skv, kv_lo=0, kv_hi=-1):
     """Key ranges the block-sparse kernel walks, per (mask head, query segment), as the device built them.
 
@@ -466,17 +581,7 @@ def block_sparse_runs(block_mask, Skv, kv_lo=0, kv_hi=-1):
     if block_mask.ndim == 2:
         block_mask = block_mask.unsqueeze(0)
     Hm, nQ, nK = block_mask.shape
-    kv_hi = Skv if kv_hi < 0 else kv_hi
-    kv_block = (kv_hi - kv_lo) // nK
-    lib = _lib.load()
-    ws_bytes = lib.pa_blocksparse_workspace_bytes(Hm, nQ, nK)
-    ws = torch.zeros((ws_bytes + 3) // 4, dtype=torch.int32, device=block_mask.device)
-    mask_u8 = block_mask.contiguous().view(torch.uint8)
-    with torch.cuda.device(block_mask.device):
-        rc = lib.pa_blocksparse_build_runs(
-            _ptr(mask_u8), Hm, nQ, nK, Skv, kv_lo, kv_block, _ptr(ws), ws_bytes, _stream_ptr(block_mask.device)
-        )
-    _lib.check(rc, "pa_blocksparse_build_runs")
+    ws = block_sparse_key_runs(block_mask, Skv, kv_lo, kv_hi)
     nseg, cap = nQ + 2, nK // 2 + 3
     count = ws[: Hm * nseg].view(Hm, nseg)
     ranges = ws[Hm * nseg : Hm * nseg + Hm * nseg * cap * 2].view(Hm, nseg, cap, 2)

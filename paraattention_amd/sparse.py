@@ -22,8 +22,11 @@ def struct_sparse_attn_func(
     sparse_range_query=None,
     sparse_range_key_value=None,
     print_attn_weight_means=False,
+    runs_cache=None,
 ):
-    """Signature of the reference's ``struct_sparse_attn_func`` (sparse_attn.py:285-311).
+    """Signature of the reference's ``struct_sparse_attn_func`` (sparse_attn.py:285-311), plus ``runs_cache``:
+    a dict in which the key ranges extracted from the mask are kept, so that a mask that serves many calls
+    (``StructSparseAttnMode`` passes its own) is scanned once per key length and not once per call.
 
     ``sparse_mask`` is the reference's 2-D bool [nQ,nK]; a 3-D [H,nQ,nK] mask (one
     per head) is accepted as well.  Returns the output only, like the reference
@@ -49,8 +52,20 @@ def struct_sparse_attn_func(
     assert 0 <= kv_lo <= kv_hi <= s_kv, f"sparse_range_key_value must be in [0, {s_kv}], got {(kv_lo, kv_hi)}"
     assert (q_hi - q_lo) % sparse_mask.shape[-2] == 0, "sparse_mask must divide the query dimension"
     assert (kv_hi - kv_lo) % sparse_mask.shape[-1] == 0, "sparse_mask must divide the key/value dimension"
-    mask = sparse_mask.to(device=query.device, dtype=torch.bool)
-    out, _ = ops.attention_forward_block_sparse(query, key, value, mask, q_lo, q_hi, kv_lo, kv_hi, scale=scale)
+    if runs_cache is None:
+        mask = sparse_mask.to(device=query.device, dtype=torch.bool)
+        out, _ = ops.attention_forward_block_sparse(query, key, value, mask, q_lo, q_hi, kv_lo, kv_hi, scale=scale)
+        return out
+    # the mask's content is identified by the tensor and its version counter (in-place edits bump it)
+    tag = (id(sparse_mask), sparse_mask._version, query.device, s_kv, kv_lo, kv_hi)
+    runs = runs_cache.get(tag)
+    if runs is None:
+        mask = sparse_mask.to(device=query.device, dtype=torch.bool)
+        runs = ops.block_sparse_key_runs(mask, s_kv, kv_lo, kv_hi)
+        runs_cache.clear()  # one mask, one key length at a time: no pile of stale entries
+        runs_cache[tag] = runs
+    shape = (1, *sparse_mask.shape) if sparse_mask.ndim == 2 else tuple(sparse_mask.shape)
+    out, _ = ops.attention_forward_block_sparse_runs(query, key, value, runs, shape[0], shape[1], shape[2], q_lo, q_hi, scale=scale)
     return out
 
 
@@ -67,7 +82,8 @@ class StructSparseAttnMode(_SdpaMode):
         super().__init__()
         self._sparse = dict(sparse_mask=sparse_mask, sparse_range_query=sparse_range_query,
                             sparse_range_key_value=sparse_range_key_value,
-                            print_attn_weight_means=print_attn_weight_means)
+                            print_attn_weight_means=print_attn_weight_means,
+                            runs_cache={} if sparse_mask is not None else None)
 
     def _call(self, *args, **kwargs):
         return struct_sparse_attn_func(*args, **kwargs, **self._sparse)

@@ -26,7 +26,9 @@ def _check(out, lse, ref_out, ref_lse, what=""):
     assert (err <= tol).all(), f"{what}: out max err {err.max():.4g} (worst excess {(err - tol).max():.4g})"
     if lse is not None:
         lse = lse.cpu().numpy().astype(np.float64)
-        lerr = np.abs(lse - np.asarray(ref_lse, dtype=np.float64))
+        ref_lse = np.asarray(ref_lse, dtype=np.float64)
+        with np.errstate(invalid="ignore"):
+            lerr = np.where(lse == ref_lse, 0.0, np.abs(lse - ref_lse))  # -inf against -inf (a row that keeps nothing) is exact
         assert lse.dtype == np.float64 and (lerr <= LSE_ATOL).all(), f"{what}: lse max err {lerr.max():.4g}"
 
 
@@ -226,6 +228,74 @@ def test_key_mask_and_sparse_kv(cuda):
         _check(out, None, ref_out, None, "sparse_kv")
         out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), m[:, None, None, :].to(cuda))
         _check(out, lse, ref_out, ref_lse, "key mask")
+
+
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_general_masks_vs_f64(cuda, D, dtype):
+    """attn_mask as the reference's dense ops take it (src/para_attn/ops/__init__.py:78-87, 215-223): boolean or
+    additive, any shape that broadcasts to [B,H,Sq,Skv] with torch's alignment of trailing dimensions.  Rows that
+    keep nothing give out = 0, lse = -inf (the oracle's convention); tiles in which a row keeps nothing at all
+    precede kept ones.  Every case against the fp64 oracle with the mask expanded."""
+    B, H, Sq, Skv = 2, 3, 150, 333
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=41, dtype=dtype)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    g = torch.Generator().manual_seed(8)
+    op = torch.ops.para_attn.attention_forward_with_lse
+    qn, kn, vn = q.float().numpy(), k.float().numpy(), v.float().numpy()
+    shapes = [(B, H, Sq, Skv), (1, 1, Sq, Skv), (Sq, Skv), (B, 1, Sq, Skv), (H, 1, Skv), (B, 1, 1, Skv), (Skv,), (1, H, Sq, 1)]
+    for shape in shapes:
+        keep = torch.rand(shape, generator=g) < 0.4
+        if len(shape) >= 2 and shape[-2] == Sq and shape[-1] == Skv:
+            keep[..., 3, :] = False        # a row that keeps nothing
+            keep[..., 5, :200] = False     # a row whose first three tiles are empty
+        ref_out, ref_lse = oattn.sdpa_lse_f64(qn, kn, vn, None, np.broadcast_to(keep.numpy(), (B, H, Sq, Skv)))
+        out, lse = op(qd, kd, vd, keep.to(cuda))
+        _check(out, lse, ref_out, ref_lse, f"bool mask {shape}")
+        assert torch.equal(torch.ops.para_attn.attention_forward(qd, kd, vd, keep.to(cuda)), out)
+        # the same mask as an additive one (0 / -inf), in fp32 and in the activation type
+        for mdt in (torch.float32, dtype):
+            bias = torch.zeros(keep.shape, dtype=mdt).masked_fill_(~keep, float("-inf"))
+            out_a, lse_a = op(qd, kd, vd, bias.to(cuda))
+            _check(out_a, lse_a, ref_out, ref_lse, f"additive -inf mask {shape} {mdt}")
+    # a finite bias: scores + bias before the softmax
+    bias = torch.randn(B, 1, Sq, Skv, generator=g)
+    s = np.einsum("bhqd,bhkd->bhqk", qn.astype(np.float64), kn.astype(np.float64)) / np.sqrt(D) + bias.numpy().astype(np.float64)
+    m = s.max(-1, keepdims=True)
+    pw = np.exp(s - m)
+    ref_out = (pw @ vn.astype(np.float64)) / pw.sum(-1, keepdims=True)
+    ref_lse = (m + np.log(pw.sum(-1, keepdims=True)))[..., 0]
+    out, lse = op(qd, kd, vd, bias.to(cuda))
+    _check(out, lse, ref_out, ref_lse, "finite additive bias")
+    # torch's own CPU SDPA agrees on the same additive mask (independent of the oracle's formula)
+    t_out, t_lse = oattn.sdpa_lse_torch_cpu(q, k, v, attn_mask=bias.to(dtype).expand(B, H, Sq, Skv).contiguous())
+    out_b, lse_b = op(qd, kd, vd, bias.to(dtype).to(cuda))
+    _check(out_b, lse_b, t_out.float().numpy(), t_lse.numpy(), "finite additive bias, torch CPU")
+    with pytest.raises(ValueError):
+        op(qd, kd, vd, torch.ones(B, Skv, dtype=torch.bool, device=cuda))  # [2,333] is not [Sq,Skv]
+
+
+def test_key_masks_take_the_fast_kernels_when_prefixes(cuda, tuning):
+    """A key-only boolean mask is scanned on the device: prefixes run the dense kernels with per-batch key counts
+    (here with the key-split tail and the score bound in play), anything else the per-score kernel; both give the
+    oracle's result and neither reads the mask on the host."""
+    tuning("bound", 1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    B, H, D = 2, 4, 128
+    Sq, Skv = (cus // (B * H) + 3) * 256 - 19, 64 * 40 + 37
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=43)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    lens = torch.tensor([Skv - 3, 900])
+    prefix = torch.arange(Skv)[None, :] < lens[:, None]
+    scattered = prefix.clone()
+    scattered[1, 10] = False
+    scattered[1, 2000] = True
+    rows = torch.cat([torch.arange(0, 30), torch.arange(Sq - 300, Sq, 7)])
+    for name, m in (("prefix", prefix), ("scattered", scattered)):
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), k.float().numpy(), v.float().numpy(), None, m[:, None, None, :].numpy())
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, m[:, None, None, :].to(cuda))
+        _check(out[:, :, rows.to(cuda)], lse[:, :, rows.to(cuda)], ref_out, ref_lse, name)
+        assert torch.isfinite(lse).all()
 
 
 @pytest.mark.parametrize("D", [128, 64])

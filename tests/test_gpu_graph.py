@@ -10,14 +10,17 @@ from oracle import inputs
 pytestmark = pytest.mark.gpu
 
 
-def _eager(q, kb, vb, prev, cur):
+def _eager(q, kb, vb, prev, cur, key_mask):
     out, lse = torch.ops.para_attn.attention_forward_with_lse(q, kb[0], vb[0])
+    # masked calls: whether the key mask is a prefix is decided on the device, inside the captured work
+    mo, ml = torch.ops.para_attn.attention_forward_with_lse(q, kb[0], vb[0], key_mask)
+    so = torch.ops.para_attn.attention_forward_sparse_kv(q, kb[0], vb[0], key_mask.expand(-1, -1, q.shape[2], -1))
     ro, rl = paraattention_amd.ring_sweep(q, kb, vb, fused=True)
     uo, ul = paraattention_amd.ring_sweep(q, kb, vb, fused=False)
     ratio = torch.ops.para_attn.fbcache_residual_diff(prev, cur)
     applied = torch.ops.para_attn.fbcache_apply_residual(prev, cur)
     tv = torch.ops.para_attn.taylorseer_value([cur, prev], 2, prev)
-    return [out, lse, ro, rl, uo, ul, ratio, applied, tv]
+    return [out, lse, ro, rl, uo, ul, ratio, applied, tv, mo, ml, so]
 
 
 def test_graph_replays_match_eager(cuda):
@@ -29,15 +32,19 @@ def test_graph_replays_match_eager(cuda):
     kb = [t.contiguous().to(cuda) for t in k.split(2600, 2)]
     vb = [t.contiguous().to(cuda) for t in v.split(2600, 2)]
     prev, cur = (t.to(cuda) for t in inputs.fbcache_pair((1, 700, 512), seed=2))
-    _eager(q, kb, vb, prev, cur)  # warm-up outside capture (library load, function attributes)
+    key_mask = (torch.arange(2600)[None, None, None, :] < 2000).to(cuda)  # a prefix at capture time
+    _eager(q, kb, vb, prev, cur, key_mask)  # warm-up outside capture (library load, function attributes)
+    key_mask[..., 5] = False
+    _eager(q, kb, vb, prev, cur, key_mask)  # and the per-score kernel's
+    key_mask[..., 5] = True
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
-        _eager(q, kb, vb, prev, cur)
+        _eager(q, kb, vb, prev, cur, key_mask)
         torch.cuda.synchronize()
         with torch.cuda.graph(graph, stream=side):
-            captured = _eager(q, kb, vb, prev, cur)
+            captured = _eager(q, kb, vb, prev, cur, key_mask)
     torch.cuda.synchronize()
     g = torch.Generator().manual_seed(5)
     for rep in range(4):
@@ -45,10 +52,12 @@ def test_graph_replays_match_eager(cuda):
             q.copy_(torch.randn(q.shape, generator=g).bfloat16())
             kb[1].copy_(torch.randn(kb[1].shape, generator=g).bfloat16())
             cur.copy_((prev.float().cpu() + 0.05 * (rep + 1) * torch.randn(prev.shape, generator=g)).bfloat16())
+            # the mask changes between replays: a shorter prefix, then a scattered mask, then a prefix again
+            key_mask.copy_(((torch.arange(2600) < 2000 - 300 * rep) ^ (torch.arange(2600) == 7 if rep == 2 else torch.zeros(2600, dtype=torch.bool)))[None, None, None, :])
         graph.replay()
         torch.cuda.synchronize()
         got = [t.clone() for t in captured]
-        want = _eager(q, kb, vb, prev, cur)
+        want = _eager(q, kb, vb, prev, cur, key_mask)
         torch.cuda.synchronize()
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), f"replay {rep}: output {i} differs from the eager run"

@@ -122,3 +122,38 @@ def test_in_batch_ring_and_ulysses_on_one_rank(cuda):
     folded = qs.permute(1, 0, 2, 3).reshape(1, H, B * Sq, D)
     assert folded.data_ptr() == qs.data_ptr()
     assert torch.equal(paraattention_amd.in_batch_attn_func(qs, ks, vs), out)
+
+
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_torch_ring_loop_calls_the_op(cuda, tmp_path, is_causal):
+    """torch's own ring loop with this package's op, the call the reference makes
+    (src/para_attn/para_attn_interface.py:164-197: _templated_ring_attention(mesh, seq_dim,
+    para_attn_ops.attention_forward_with_lse, q, k, v, attn_mask=, dropout_p=, is_causal=, scale=) with load
+    balancing off and fp32 merging).  On a group of one rank the loop issues no collective: it calls the op once
+    as op(q, k, v, is_causal=..., **kwargs), unpacks (out, lse, *rest), passes both through _SDPAMerger and casts
+    back, so the result must be the op's own, bit for bit."""
+    import torch.distributed as dist
+    from torch.distributed.tensor.experimental._context_parallel import _attention as tra
+
+    if dist.is_initialized():
+        pytest.skip("a default process group already exists in this process")
+    dist.init_process_group("gloo", store=dist.FileStore(str(tmp_path / "rendezvous"), 1), rank=0, world_size=1)
+    saved = (tra._cp_options.enable_load_balance, tra._cp_options.convert_to_f32, tra._cp_options.rotate_method)
+    try:
+        tra._cp_options.enable_load_balance = False
+        tra._cp_options.convert_to_f32 = True
+        tra._cp_options.rotate_method = tra._RotateMethod.ALL_TO_ALL
+        q, k, v = inputs.qkv(1, 3, 300, 300, 128, seed=21)
+        qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+        out, lse = tra._templated_ring_attention(dist.group.WORLD, 2, torch.ops.para_attn.attention_forward_with_lse,
+                                                 qd, kd, vd, attn_mask=None, dropout_p=0.0, is_causal=is_causal, scale=None)
+        want_out, want_lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, is_causal=is_causal)
+        assert out.dtype == torch.bfloat16 and torch.equal(out, want_out)
+        assert lse.dtype == torch.float32 and torch.equal(lse.reshape(want_lse.shape), want_lse)
+        keep = oattn.causal_keep(300, 300) if is_causal else None
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, keep)
+        np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+        np.testing.assert_allclose(lse.reshape(want_lse.shape).cpu().numpy(), ref_lse, atol=1e-3)
+    finally:
+        (tra._cp_options.enable_load_balance, tra._cp_options.convert_to_f32, tra._cp_options.rotate_method) = saved
+        dist.destroy_process_group()

@@ -111,6 +111,44 @@ def test_sparse_ranges_with_dense_margins(cuda):
     np.testing.assert_allclose(dense.float().cpu().numpy(), ref_dense, atol=2e-2, rtol=2e-2)
 
 
+def test_prebuilt_runs_entry(cuda):
+    """A mask that serves many calls is scanned once: attention_forward_block_sparse_runs with the ranges from
+    block_sparse_key_runs gives bit for bit what attention_forward_block_sparse gives, for shared and per-head
+    masks, with margins, on keys of another content; the mode caches the ranges and follows in-place edits."""
+    B, H, D = 1, 3, 128
+    Sq, Skv = 16 + 4 * 128 + 40, 24 + 6 * 64 + 8
+    q_range, kv_range = (16, 16 + 512), (24, 24 + 384)
+    q, k, v = (t.to(cuda) for t in inputs.qkv(B, H, Sq, Skv, D, seed=5))
+    g = torch.Generator().manual_seed(9)
+    for shape in ((4, 6), (H, 4, 6)):
+        bm = torch.rand(shape, generator=g) < 0.5
+        bm[..., 0] = True
+        want_out, want_lse = torch.ops.para_attn.attention_forward_block_sparse(q, k, v, bm.to(cuda), *q_range, *kv_range)
+        runs = torch.ops.para_attn.block_sparse_key_runs(bm.to(cuda), Skv, *kv_range)
+        hm = 1 if bm.ndim == 2 else H
+        for kk, vv in ((k, v), (v, k)):  # the ranges depend on the mask only
+            w_out, w_lse = torch.ops.para_attn.attention_forward_block_sparse(q, kk, vv, bm.to(cuda), *q_range, *kv_range)
+            out, lse = torch.ops.para_attn.attention_forward_block_sparse_runs(q, kk, vv, runs, hm, 4, 6, *q_range)
+            assert torch.equal(out, w_out) and torch.equal(lse, w_lse)
+        with pytest.raises(ValueError):
+            torch.ops.para_attn.attention_forward_block_sparse_runs(q, k, v, runs[:10], hm, 4, 6, *q_range)
+    bm = torch.rand((4, 6), generator=g) < 0.5
+    bm[:, 0] = True
+    with paraattention_amd.StructSparseAttnMode(sparse_mask=bm, sparse_range_query=q_range, sparse_range_key_value=kv_range) as mode:
+        cache = mode._sparse["runs_cache"]
+        o1 = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+        (held,) = cache.values()
+        o2 = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+        assert next(iter(cache.values())) is held and torch.equal(o1, o2)  # second call: no new scan
+        want, _ = torch.ops.para_attn.attention_forward_block_sparse(q, k, v, bm.to(cuda), *q_range, *kv_range)
+        assert torch.equal(o1, want)
+        bm[1] = ~bm[1]
+        bm[1, 0] = True  # edited in place: the version counter moves, the ranges are rebuilt
+        o3 = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+        want3, _ = torch.ops.para_attn.attention_forward_block_sparse(q, k, v, bm.to(cuda), *q_range, *kv_range)
+        assert torch.equal(o3, want3) and len(cache) == 1 and next(iter(cache.values())) is not held
+
+
 def test_row_without_kept_block(cuda):
     # the reference asserts out on such a row (torch _SDPAMerger.results() with nothing merged);
     # the kernel defines it: out = 0, lse = -inf

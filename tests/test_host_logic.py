@@ -123,13 +123,27 @@ def test_row_view_helper():
     assert ops._as_rows(t.transpose(0, 1)) is None
 
 
-def test_key_keep_vector():
-    B, Skv = 2, 10
+def test_mask_broadcasting_follows_torch():
+    """attn_mask is read as F.scaled_dot_product_attention reads it (trailing dimensions aligned with
+    [B,H,Sq,Skv], src/para_attn/ops/__init__.py:215-223): a 2-D mask is [Sq,Skv], never a per-batch key mask."""
+    from paraattention_amd import _lib
+
+    B, H, Sq, Skv = 2, 3, 5, 10
     m = torch.rand(B, Skv) < 0.5
-    assert torch.equal(ops._key_keep_vector(m[:, None, None, :], B, Skv), m)
-    assert torch.equal(ops._key_keep_vector(m[:1, None, None, :], B, Skv), m[:1].expand(B, Skv))
-    assert ops._key_keep_vector(torch.zeros(B, 1, 5, Skv, dtype=torch.bool), B, Skv) is None  # per-query mask
-    assert ops._key_keep_vector(torch.zeros(B, 1, 1, Skv), B, Skv) is None  # additive mask
+    t, kind, st = ops._broadcast_mask(m[:, None, None, :], B, H, Sq, Skv, torch.bfloat16)
+    assert kind == _lib.PA_MASK_BOOL and list(st) == [Skv, 0, 0, 1]
+    t, kind, st = ops._broadcast_mask(torch.zeros(Sq, Skv), B, H, Sq, Skv, torch.bfloat16)
+    assert kind == _lib.PA_MASK_F32 and list(st) == [0, 0, Skv, 1] and t.shape == (1, 1, Sq, Skv)
+    t, kind, st = ops._broadcast_mask(torch.zeros(H, 1, Skv, dtype=torch.bfloat16), B, H, Sq, Skv, torch.bfloat16)
+    assert kind == _lib.PA_MASK_ACT and list(st) == [0, Skv, 0, 1]
+    t, kind, st = ops._broadcast_mask(torch.zeros(B, H, Sq, Skv, dtype=torch.float16), B, H, Sq, Skv, torch.bfloat16)
+    assert kind == _lib.PA_MASK_F32 and t.dtype == torch.float32  # another float type than the activations': widened
+    with pytest.raises(ValueError):
+        ops._broadcast_mask(m, B, H, Sq, Skv, torch.bfloat16)  # [2,10] against Sq = 5: does not broadcast
+    with pytest.raises(ValueError):
+        ops._broadcast_mask(torch.zeros(Sq, Skv, dtype=torch.int32), B, H, Sq, Skv, torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops._broadcast_mask(torch.zeros(1, 1, 1, 1, Skv), B, H, Sq, Skv, torch.bfloat16)
 
 
 def test_merger_refuses_partial_mode():
