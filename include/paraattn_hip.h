@@ -57,6 +57,8 @@ PA_API const char* pa_last_error(void);
  *   "no_split"     PARAATTN_NO_SPLIT=1      1: no key-split tail
  *   "no_xcd_order" PARAATTN_NO_XCD_ORDER=1  1: block-sparse workgroups in plain order
  *   "bound"        PARAATTN_BOUND=0|1       0 / 1: never / always compute the score bound, -1 = by size
+ *   "stream"       PARAATTN_STREAM=0|1      0 / 1: never / wherever possible the kernel with resident workgroups, -1 = by shape
+ *   "stream_even"  PARAATTN_STREAM_EVEN=0|1 that kernel's tail cut into shares that begin at the same keys / into equal ranges, -1 = by size
  * Returns PA_ERR_INVALID for an unknown name or value.
  */
 PA_API int pa_set_tuning(const char* name, int value);
@@ -192,6 +194,32 @@ PA_API int pa_attn_fwd_accumulate(const void* q, const void* k, const void* v, f
                            const int64_t v_strides[3], const int64_t out_strides[3], float scale,
                            const int32_t* kv_len, int first, void* workspace,
                            size_t workspace_bytes, void* stream);
+
+/*
+ * A whole same-GPU ring sweep in one launch: attention of q against the
+ * concatenation of n_blocks key/value blocks that lie at separate addresses
+ * (the blocks a ring pass visits, src/para_attn/para_attn_interface.py:164-197:
+ * one attention call and one _SDPAMerger.step per block in torch's
+ * _templated_ring_attention).  The kernel walks the blocks as one key sequence
+ * and carries the softmax state (running maximum, sum, output) across them in
+ * registers, so neither the per-block outputs nor the fp32 running pair of
+ * pa_attn_fwd_accumulate exist.  Result: out and lse of attention over all
+ * n_blocks * block_len keys.
+ *
+ * k_blocks, v_blocks: host arrays of n_blocks (1..16) device pointers to
+ * [B,H,block_len,D] tensors that share k_strides / v_strides; head_dim 128,
+ * each block below 4 GiB per (batch, head).  Otherwise PA_ERR_UNSUPPORTED (run
+ * pa_attn_fwd_accumulate per block instead).  workspace: as for
+ * pa_attn_fwd_lse_ws, of pa_attn_fwd_sweep_workspace_bytes() bytes; may be NULL.
+ */
+PA_API int pa_attn_fwd_sweep(const void* q, const void* const* k_blocks, const void* const* v_blocks, int n_blocks,
+                      int block_len, void* out, float* lse, int dtype, int B, int H, int Sq, int D,
+                      const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                      const int64_t out_strides[3], float scale, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+PA_API size_t pa_attn_fwd_sweep_workspace_bytes(int B, int H, int Sq, int n_blocks, int block_len, int D,
+                                         const int64_t k_strides[3], const int64_t v_strides[3]);
 
 /*
  * Bytes of workspace pa_attn_fwd_lse_ws and pa_attn_fwd_accumulate can use for this problem on the current

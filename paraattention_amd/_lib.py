@@ -69,6 +69,11 @@ SIGNATURES = {
          _i, _vp, _sz, _vp],
     ),
     "pa_attn_fwd_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _strides, _strides]),
+    "pa_attn_fwd_sweep": (
+        _i,
+        [_vp, _ptrs, _ptrs, _i, _i, _vp, _vp, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _sz, _vp],
+    ),
+    "pa_attn_fwd_sweep_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _strides, _strides]),
     "pa_attn_fwd_blocksparse": (
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f,
@@ -141,7 +146,7 @@ def check(rc, what):
 
 def set_tuning(name, value):
     """Set one tuning / test knob of the attention launches (pa_set_tuning in the header): "no_pipe", "bm",
-    "no_split", "no_xcd_order", "bound".  The PARAATTN_* environment variables only give the initial values."""
+    "no_split", "no_xcd_order", "bound", "stream", "stream_even".  The PARAATTN_* environment variables only give the initial values."""
     check(load().pa_set_tuning(name.encode(), int(value)), "pa_set_tuning")
 
 

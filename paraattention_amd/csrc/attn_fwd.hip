@@ -45,6 +45,25 @@ constexpr float LN2 = 0.6931471805599453f;
 // many powers of two; below that the accumulators keep their scale (P <= 2^8).
 constexpr float RESCALE_SLACK = 8.0f;
 
+// Work plan of attn_fwd_d128_stream_kernel.  The launch has G workgroups of 256 query rows that stay resident.
+// A piece is one query tile of one (batch, head) with its L key tiles.  Workgroup g first computes the R whole
+// pieces g, g + G, ..., all workgroups sweeping the keys in step (so a K/V tile is fetched once per L2 and
+// round); what is left, fewer than G pieces, is a list of (n_pieces - R G) L key-tile steps cut into Gt equal
+// ranges, one for each of the first Gt workgroups.  A range that does not cover a whole piece leaves a
+// normalised fp32 partial result and its LSE in the workspace (at most two per workgroup: row 2g for a share
+// that begins inside a piece, 2g + 1 for one that begins a piece but does not finish it), which
+// attn_stream_merge_kernel folds.  Gt = G cuts the tail evenly; Gt = (pieces left) x s cuts every piece
+// left into s shares that begin at the same keys.
+// The keys of a piece may come in nseg segments of seg_len keys each (the blocks of a ring sweep), each with
+// its own base pointer and the strides of AttnParams.
+constexpr int MAX_KEY_SEGS = 16;
+struct StreamPlan {
+  int G, R, Gt, L, n_pieces;
+  int nseg, seg_len, tps;  // key segments, keys and key tiles per segment
+  const void* kseg[MAX_KEY_SEGS];
+  const void* vseg[MAX_KEY_SEGS];
+};
+
 struct AttnParams {
   const void* q;
   const void* k;
@@ -95,9 +114,11 @@ struct AttnParams {
   // the device by an earlier launch of the same stream, e.g. whether a key mask is a prefix)
   const int* gate;
   int gate_want;
+  StreamPlan st;  // attn_fwd_d128_stream_kernel only
 };
 
 constexpr int MASK_NONE = 0, MASK_BOOL = 1, MASK_F32 = 2, MASK_ACT = 3;
+
 
 template <int D>
 struct Smem {
@@ -928,13 +949,24 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   int row_begin, row_end;
   TileIter it;
   decode_block<SPARSE>(p, qt, head, batch, row_begin, row_end, it);
+  // Keys in segments (the blocks of a ring sweep, StreamPlan::kseg / vseg): the sweep below runs once per
+  // segment, with the softmax state carried over in registers.  A key share of a split piece is then a run of
+  // whole segments; with one segment it is a range of key tiles.
+  int seg_lo = 0, seg_hi = 1;
   if constexpr (!SPARSE) {
+    const int nseg = p.st.nseg > 1 ? p.st.nseg : 1;
+    seg_hi = nseg;
     if (piece_slot >= 0) {
-      const int len = it.end;
-      const int nkt = (len + BN - 1) / BN;
       const int piece = piece_slot / p.split_tiles;
-      const int t0 = (int)((int64_t)piece * nkt / p.split_s), t1 = (int)((int64_t)(piece + 1) * nkt / p.split_s);
-      it.init_range(t0 * BN, t1 * BN < len ? t1 * BN : len);
+      if (nseg > 1) {
+        seg_lo = piece * nseg / p.split_s;
+        seg_hi = (piece + 1) * nseg / p.split_s;
+      } else {
+        const int len = it.end;
+        const int nkt = (len + BN - 1) / BN;
+        const int t0 = (int)((int64_t)piece * nkt / p.split_s), t1 = (int)((int64_t)(piece + 1) * nkt / p.split_s);
+        it.init_range(t0 * BN, t1 * BN < len ? t1 * BN : len);
+      }
     }
   }
 
@@ -962,18 +994,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   // the logical chunk that the swizzle maps there.  Inline assembly on purpose: the compiler
   // keeps no account of these copies, so LDS reads that follow do not wait for them; completion
   // is awaited by hand (vmcnt(0)) in front of the barrier.
-  auto make_rsrc = [&](const char* base, uint32_t row_bytes) {
+  auto make_rsrc = [&](const char* base, uint32_t row_bytes, int n_keys) {
     u32x4 r;
     const uint64_t a = (uint64_t)base;
-    const uint64_t nbytes = (uint64_t)(p.Skv - 1) * row_bytes + 256;  // start of the last row + one row
+    const uint64_t nbytes = (uint64_t)(n_keys - 1) * row_bytes + 256;  // start of the last row + one row
     r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
     r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
     r[2] = __builtin_amdgcn_readfirstlane((uint32_t)nbytes);
     r[3] = 0x00020000u;
     return r;
   };
-  const u32x4 krs = make_rsrc(kbytes, ks_bytes);
-  const u32x4 vrs = make_rsrc(vbytes, vs_bytes);
+  u32x4 krs = make_rsrc(kbytes, ks_bytes, p.Skv);
+  u32x4 vrs = make_rsrc(vbytes, vs_bytes, p.Skv);
   const int dma_row = 4 * wave + (lane >> 4);
   const int dma_pc = lane & 15;
   const uint32_t k_off0 = dma_row * ks_bytes + 16 * (dma_pc ^ (dma_row & 15));
@@ -1042,10 +1074,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       nv = 0;
     }
   };
-  pull(n_cur, v_cur);
-  pull(n_nxt, v_nxt);
-  pull(n_nx2, v_nx2);
-  bool have = n_cur != OOB;
+  bool have = false;
 
   // -inf on the keys past the end of a ragged tile: register r of this lane is key
   // 8*(r/4) + r%4 + 4*hh of the first half (+32 for the second); constants against one per-lane
@@ -1079,34 +1108,6 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   float mx = 0.f;     // row maximum of S(j), masked, unscaled
 #pragma unroll
   for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
-
-  // ---- prologue: K0, V0, K1 copies; S(0) and its row maximum ---------------------------------
-  if (have) {
-#pragma unroll
-    for (int i = 0; i < IPW; ++i) dma_k1(0, n_cur, i);
-#pragma unroll
-    for (int i = 0; i < IPW; ++i) dma_v1(0, n_cur, i);
-#pragma unroll
-    for (int i = 0; i < IPW; ++i) dma_k1(1, n_nxt, i);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-#pragma unroll
-    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(sK, 0, dc);
-#pragma unroll
-    for (int dc = 0; dc < DC; ++dc) {
-      sn0 = T::mfma32(f[dc], qf[dc], sn0);
-      f[dc] = read_k(sK, 1, dc);
-    }
-#pragma unroll
-    for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
-    if (v_cur < BN || on_diagonal(n_cur)) mask_tail(sn0, sn1, v_cur, n_cur);
-    if constexpr (!BOUNDED) {
-      float m2 = fmaxf(sn0[0], sn1[0]);
-#pragma unroll
-      for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
-      mx = across(m2);
-    }
-  }
 
   // One iteration; PAR = buffer of tile j (K(j+1) sits in the other K buffer).
   auto tile_step = [&](auto PAR) {
@@ -1242,12 +1243,61 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     have = n_cur != OOB;
   };
 
-  while (have) {
-    tile_step(std::integral_constant<int, 0>{});
-    if (!have) break;
-    tile_step(std::integral_constant<int, 1>{});
+  // The keys' segments are swept one after the other, the pipeline drained in between (carrying it across, with
+  // the copies' descriptors following their tile's segment, was measured: the bookkeeping that adds to every
+  // iteration costs 4.5 % of the sweep, the drains it saves 2 %).
+  for (int seg = seg_lo; seg < seg_hi; ++seg) {
+    if constexpr (!SPARSE) {
+      if (p.st.nseg > 1) {  // this segment's keys and values, all of them
+        const int64_t koff = (batch * p.ks_b + head * p.ks_h) * 2, voff = (batch * p.vs_b + head * p.vs_h) * 2;
+        krs = make_rsrc((const char*)p.st.kseg[seg] + koff, ks_bytes, p.st.seg_len);
+        vrs = make_rsrc((const char*)p.st.vseg[seg] + voff, vs_bytes, p.st.seg_len);
+        it.init_dense(p.st.seg_len);
+        if (seg > seg_lo) __syncthreads();  // everybody has left the previous segment's last tiles
+      }
+    }
+    pull(n_cur, v_cur);
+    pull(n_nxt, v_nxt);
+    pull(n_nx2, v_nx2);
+    have = n_cur != OOB;
+    if (seg > seg_lo) {  // the scores left over from the previous segment's last, absent tile
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+    }
+    // ---- prologue: K0, V0, K1 copies; S(0) and its row maximum ---------------------------------
+    if (have) {
+#pragma unroll
+      for (int i = 0; i < IPW; ++i) dma_k1(0, n_cur, i);
+#pragma unroll
+      for (int i = 0; i < IPW; ++i) dma_v1(0, n_cur, i);
+#pragma unroll
+      for (int i = 0; i < IPW; ++i) dma_k1(1, n_nxt, i);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(sK, 0, dc);
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        sn0 = T::mfma32(f[dc], qf[dc], sn0);
+        f[dc] = read_k(sK, 1, dc);
+      }
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
+      if (v_cur < BN || on_diagonal(n_cur)) mask_tail(sn0, sn1, v_cur, n_cur);
+      if constexpr (!BOUNDED) {
+        float m2 = fmaxf(sn0[0], sn1[0]);
+#pragma unroll
+        for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
+        mx = across(m2);
+      }
+    }
+    while (have) {
+      tile_step(std::integral_constant<int, 0>{});
+      if (!have) break;
+      tile_step(std::integral_constant<int, 1>{});
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the segment, or the wavefront, ends
   }
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the wavefront ends
 
   // ---- epilogue -----------------------------------------------------------------------------------
   float l_tot;
@@ -1671,6 +1721,579 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// head_dim 128, resident workgroups (StreamPlan above): the two-tile pipeline of
+// attn_fwd_d128_pipe_kernel<.., 8> run over a list of pieces per workgroup as ONE stream of key
+// tiles.  The copies of K(j+2) and V(j+1) and the scores S(j+1) simply belong to the next piece when
+// tile j is the last of its piece, so the next piece's first tiles, its Q fragments (fetched into the
+// registers the finished piece's Q has left, one iteration ahead) and its first score tile are all
+// under way while the current piece's last tiles are computed; the output of a finished piece is
+// stored from inside the loop.  What a launch of one workgroup per piece pays per piece (Q load,
+// first copies, S(0), output drain: 5-10 us against 1.7 us per key tile) is hidden behind the
+// neighbouring pieces' MFMA work.  Dense, not causal, no per-batch key counts.
+// ---------------------------------------------------------------------------------------------
+template <typename T, bool BOUNDED>
+__global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const AttnParams p) {
+  typedef typename T::vec8 vec8;
+  constexpr int NW = 8, DC = 8, DB = 4;
+  constexpr int IPW = 16 / NW;  // copy instructions per wavefront and K (V) tile
+  constexpr int RS = 4 * NW;    // tile rows between two of them
+  if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
+  if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  char* const sK = (char*)smem;                    // [2][64][256 B]
+  char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+  const StreamPlan& sp = p.st;
+  const int wg = blockIdx.x;
+  constexpr uint32_t OOB = PIPE_OOB;
+  // What happens once per piece (a new Q, a new K/V descriptor, a finished piece's output) needs many of the
+  // kernel's arguments and little else.  Read through `p` the compiler would load them all once, ahead of the
+  // loop, and hold them in scalar registers across it (more than there are: they end up parked in vector
+  // lanes and fetched back on every iteration).  Those paths therefore read the argument block where it lies,
+  // through a pointer the compiler cannot see through, so the loads stay inside the rare branches.
+  typedef const __attribute__((address_space(4))) AttnParams* KArgs;
+  auto kargs = [&]() __attribute__((always_inline)) {
+    KArgs kp = (KArgs)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(kp));
+    return kp;
+  };
+
+  // ---- this workgroup's list of key tiles ------------------------------------------------------
+  // R whole pieces, then one range of the tail's key-tile steps, which may run over several pieces.  The
+  // generator walks items (piece, first tile, end tile) and inside an item the tiles, keeping (segment, tile
+  // in segment).
+  int tail_left = 0;  // key tiles of this workgroup's tail range still to hand out
+  if (wg < sp.Gt) {
+    const int64_t Ttail = (int64_t)(sp.n_pieces - sp.R * sp.G) * sp.L;
+    tail_left = (int)((int64_t)(wg + 1) * Ttail / sp.Gt - (int64_t)wg * Ttail / sp.Gt);
+  }
+  struct Desc {
+    int piece;    // < 0: no such tile
+    int flags;    // LAST: the item's last tile; FULL: the item is a whole piece; MID: the item begins inside a piece
+    int seg;      // key segment
+    uint32_t n0;  // first key inside the segment, or OOB
+  };
+  constexpr int LAST = 1, FULL = 2, MID = 4;
+  int g_round = -1, g_piece = 0, g_j = 0, g_kind = 0, g_jend = 0, g_seg = 0, g_jj = 0;
+  bool g_in_tail = false, g_done = false;
+  auto start_item = [&](int piece, int j0, int jend) __attribute__((always_inline)) {
+    g_piece = piece;
+    g_j = j0;
+    g_jend = jend;
+    g_kind = (j0 == 0 && jend == sp.L ? FULL : 0) | (j0 > 0 ? MID : 0);
+    g_seg = j0 / sp.tps;
+    g_jj = j0 - g_seg * sp.tps;
+  };
+  // valid keys of the tile that begins at key n0 of its segment (0 for a tile that does not exist)
+  auto valid_keys = [&](uint32_t n0) __attribute__((always_inline)) {
+    if (n0 == OOB) return 0;
+    const int left = sp.seg_len - (int)n0;
+    return left < BN ? left : BN;
+  };
+  auto advance_item = [&]() __attribute__((always_inline)) -> bool {
+    const KArgs kp = kargs();
+    const int R = kp->st.R, G = kp->st.G, L = kp->st.L;
+    if (g_round + 1 < R) {
+      ++g_round;
+      start_item(wg + g_round * G, 0, L);
+      return true;
+    }
+    if (tail_left <= 0) return false;
+    int piece, j0;
+    if (!g_in_tail) {
+      g_in_tail = true;
+      const int64_t Ttail = (int64_t)(kp->st.n_pieces - R * G) * L;
+      const int64_t ta = (int64_t)wg * Ttail / kp->st.Gt;
+      piece = R * G + (int)(ta / L);
+      j0 = (int)(ta % L);
+    } else {
+      piece = g_piece + 1;
+      j0 = 0;
+    }
+    const int n = tail_left < L - j0 ? tail_left : L - j0;
+    start_item(piece, j0, j0 + n);
+    tail_left -= n;
+    return true;
+  };
+  auto pull = [&](Desc& d) __attribute__((always_inline)) {
+    if (!g_done && g_j >= g_jend) g_done = !advance_item();
+    if (g_done) {
+      d.piece = -1; d.flags = 0; d.seg = 0; d.n0 = OOB;
+      return;
+    }
+    d.piece = g_piece;
+    d.flags = (g_j == g_jend - 1 ? LAST : 0) | g_kind;
+    d.seg = g_seg;
+    d.n0 = (uint32_t)g_jj * BN;
+    ++g_j;
+    if (++g_jj == sp.tps) {
+      g_jj = 0;
+      ++g_seg;
+    }
+  };
+  Desc cur, nxt, nx2;
+  pull(cur);
+  pull(nxt);
+  pull(nx2);
+  if (cur.piece < 0) return;  // nothing for this workgroup (before any barrier: the whole workgroup leaves)
+
+  // ---- per-piece facts ---------------------------------------------------------------------------
+  struct Where {
+    int batch, head, row_begin, row_end;
+  };
+  auto where = [&](KArgs kp, int piece) __attribute__((always_inline)) {
+    Where w;
+    const int nqt = kp->n_qtiles, H = kp->H, Sq = kp->Sq;
+    const int bh = piece / nqt;
+    const int qt = piece - bh * nqt;
+    w.head = bh % H;
+    w.batch = bh / H;
+    w.row_begin = qt * 256;
+    w.row_end = w.row_begin + 256 < Sq ? w.row_begin + 256 : Sq;
+    return w;
+  };
+  vec8 qf[DC];  // B operand of the first GEMM: the Q rows of the piece whose scores are computed next
+  auto load_q = [&](int piece) __attribute__((always_inline)) {
+    const KArgs kp = kargs();
+    const Where w = where(kp, piece);
+    int r = w.row_begin + wave * 32 + l32;
+    r = r < w.row_end ? r : w.row_end - 1;
+    const uint16_t* qp = (const uint16_t*)kp->q + w.batch * kp->qs_b + w.head * kp->qs_h + (int64_t)r * kp->qs_s + 8 * hh;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
+  };
+
+  // ---- global -> LDS copies (as in attn_fwd_d128_pipe_kernel); the descriptor follows the tile's piece and segment
+  const uint32_t ks_bytes = (uint32_t)(p.ks_s * 2), vs_bytes = (uint32_t)(p.vs_s * 2);
+  auto make_rsrc = [&](bool is_v, int seg, int piece) __attribute__((always_inline)) {
+    const KArgs kp = kargs();
+    const Where w = where(kp, piece);
+    const void* seg_base = is_v ? kp->st.vseg[seg] : kp->st.kseg[seg];
+    const int64_t sb = is_v ? kp->vs_b : kp->ks_b, sh = is_v ? kp->vs_h : kp->ks_h;
+    const uint32_t row_bytes = (uint32_t)((is_v ? kp->vs_s : kp->ks_s) * 2);
+    const uint64_t a = (uint64_t)((const uint16_t*)seg_base + w.batch * sb + w.head * sh);
+    const uint64_t nbytes = (uint64_t)(kp->st.seg_len - 1) * row_bytes + 256;  // start of the last row + one row
+    u32x4 r;
+    r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+    r[2] = __builtin_amdgcn_readfirstlane((uint32_t)nbytes);
+    r[3] = 0x00020000u;
+    return r;
+  };
+  u32x4 krs = {0, 0, 0, 0x00020000u}, vrs = {0, 0, 0, 0x00020000u};
+  int k_piece = -1, k_seg = -1, v_piece = -1, v_seg = -1;
+  auto aim_k = [&](const Desc& d) __attribute__((always_inline)) {  // point the K descriptor at the tile's piece and segment
+    if (d.piece >= 0 && (d.piece != k_piece || d.seg != k_seg)) {
+      krs = make_rsrc(false, d.seg, d.piece);
+      k_piece = d.piece;
+      k_seg = d.seg;
+    }
+  };
+  auto aim_v = [&](const Desc& d) __attribute__((always_inline)) {
+    if (d.piece >= 0 && (d.piece != v_piece || d.seg != v_seg)) {
+      vrs = make_rsrc(true, d.seg, d.piece);
+      v_piece = d.piece;
+      v_seg = d.seg;
+    }
+  };
+  const int dma_row = 4 * wave + (lane >> 4);
+  const int dma_pc = lane & 15;
+  const uint32_t k_off0 = dma_row * ks_bytes + 16 * (dma_pc ^ (dma_row & 15));
+  const uint32_t v_off0 = dma_row * vs_bytes + 16 * (dma_pc ^ (4 * (dma_row & 3)));
+  const uint32_t lds_k = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sK + wave * 1024);
+  const uint32_t lds_v = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sV + wave * 1024);
+  auto dma_k1 = [&](int buf, uint32_t n0, int i) __attribute__((always_inline)) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * ks_bytes);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_k + buf * TILE_BYTES + i * (RS * 256)), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
+  };
+  auto dma_v1 = [&](int buf, uint32_t n0, int i) __attribute__((always_inline)) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * vs_bytes);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_v + buf * TILE_BYTES + i * (RS * 256)), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
+  };
+
+  // ---- fragment read addresses (as in attn_fwd_d128_pipe_kernel) ------------------------------------
+  uint32_t ka[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) ka[dc] = l32 * 256 + 16 * ((2 * dc + hh) ^ (l32 & 15));
+  uint32_t va[DB];
+  {
+    const int g16 = lane >> 4, lg = lane & 15, r = lg >> 2, cq = lg & 3, dhalf = g16 & 1;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      va[db] = (4 * hh + r) * 256 + 16 * ((4 * db + 2 * dhalf + (cq >> 1)) ^ (4 * r)) + 8 * (cq & 1);
+  }
+  auto read_k = [&](const char* tile, int t, int dc) __attribute__((always_inline)) -> vec8 {
+    return *(const vec8*)(tile + t * 32 * 256 + ka[dc]);
+  };
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  auto read_vt = [&](const char* tile, int t, int c, int db) __attribute__((always_inline)) -> vec8 {
+    const char* a = tile + (32 * t + 16 * c) * 256 + va[db];
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + 8 * 256));
+    typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
+    s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(vec8, v);
+  };
+
+  // ---- accumulators ---------------------------------------------------------------------------
+  floatx16 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m_run = BOUNDED ? 0.f : -INFINITY, l_run = 0.f;
+  const float c = p.scale_log2;
+
+  auto mask_tail = [&](floatx16& a0, floatx16& a1, int nvalid) __attribute__((always_inline)) {
+    const int lim = nvalid - 4 * hh;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (8 * (r >> 2) + (r & 3) >= lim) a0[r] = -INFINITY;
+      if (8 * (r >> 2) + (r & 3) + 32 >= lim) a1[r] = -INFINITY;
+    }
+  };
+  auto across = [&](float x) __attribute__((always_inline)) {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+  };
+
+  // ---- output of a finished item ---------------------------------------------------------------
+  auto finish_item = [&](const Desc& d) __attribute__((always_inline)) {
+    float l_tot;
+    {
+      auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+      l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    const float lse_nat = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+    const KArgs kp = kargs();
+    const Where w = where(kp, d.piece);
+    const int my_row = w.row_begin + wave * 32 + l32;
+    float* const acc_out = kp->acc_out;
+    if (my_row < w.row_end) {
+      if (!(d.flags & FULL)) {  // a share of a piece: normalised fp32 partial + LSE into the workspace
+        const int64_t wrow = (int64_t)(2 * wg + ((d.flags & MID) ? 0 : 1)) * 256 + (my_row - w.row_begin);
+        float* wp = kp->ws_out + wrow * 128;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            float4 x = {o[db][4 * a] * inv, o[db][4 * a + 1] * inv, o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv};
+            *(float4*)(wp + 32 * db + 8 * a + 4 * hh) = x;
+          }
+        if (hh == 0) kp->ws_lse[wrow] = lse_nat;
+      } else if (acc_out != nullptr) {  // fold into the running (out, lse) pair
+        const int64_t ridx = ((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row;
+        const int acc_first = kp->acc_first;
+        float* const acc_lse = kp->acc_lse;
+        const float old = acc_first ? -INFINITY : acc_lse[ridx];
+        const float mx2 = fmaxf(old, lse_nat);
+        float w_old = 0.f, w_blk = 0.f, lse_new = -INFINITY;
+        if (mx2 > -INFINITY) {
+          const float e_old = __expf(old - mx2), e_blk = __expf(lse_nat - mx2);
+          const float den = e_old + e_blk;
+          w_old = e_old / den;
+          w_blk = e_blk / den * inv;
+          lse_new = mx2 + __logf(den);
+        }
+        float* ap = acc_out + ridx * 128;
+        uint16_t* op = kp->out ? (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h + (int64_t)my_row * kp->os_s : nullptr;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            const int d0 = 32 * db + 8 * a + 4 * hh;
+            float4 r = {0.f, 0.f, 0.f, 0.f};
+            if (!acc_first && w_old > 0.f) r = *(const float4*)(ap + d0);
+            r.x = r.x * w_old + o[db][4 * a] * w_blk;
+            r.y = r.y * w_old + o[db][4 * a + 1] * w_blk;
+            r.z = r.z * w_old + o[db][4 * a + 2] * w_blk;
+            r.w = r.w * w_old + o[db][4 * a + 3] * w_blk;
+            if (op) {
+              u32x2 x;
+              x[0] = T::pack2(r.x, r.y);
+              x[1] = T::pack2(r.z, r.w);
+              *(u32x2*)(op + d0) = x;
+            } else {
+              *(float4*)(ap + d0) = r;
+            }
+          }
+        if (hh == 0) acc_lse[ridx] = lse_new;
+      } else {
+        uint16_t* op = (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h + (int64_t)my_row * kp->os_s;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            u32x2 x;
+            x[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
+            x[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
+            *(u32x2*)(op + 32 * db + 8 * a + 4 * hh) = x;
+          }
+        float* const lse_out = kp->lse;
+        if (lse_out != nullptr && hh == 0) lse_out[((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row] = lse_nat;
+      }
+    }
+    // the next item starts from nothing
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+    m_run = BOUNDED ? 0.f : -INFINITY;
+    l_run = 0.f;
+  };
+
+  vec8 f[8];          // ring of 8 operand fragments
+  floatx16 sn0, sn1;  // S(j+1) (keys 0..31, 32..63)
+  float mx = 0.f;     // row maximum of S(j), masked, unscaled
+#pragma unroll
+  for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+
+  // ---- prologue: Q of the first piece; K0, V0, K1 copies; S(0) and its row maximum -------------------
+  load_q(cur.piece);
+  aim_k(cur);
+  aim_v(cur);
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) dma_k1(0, cur.n0, i);
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) dma_v1(0, cur.n0, i);
+  aim_k(nxt);
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) dma_k1(1, nxt.n0, i);
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(sK, 0, dc);
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) {
+    sn0 = T::mfma32(f[dc], qf[dc], sn0);
+    f[dc] = read_k(sK, 1, dc);
+  }
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
+  {
+    const int nv0 = valid_keys(cur.n0);
+    if (nv0 < BN) mask_tail(sn0, sn1, nv0);
+  }
+  if constexpr (!BOUNDED) {
+    float m2 = fmaxf(sn0[0], sn1[0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
+    mx = across(m2);
+  }
+  // the scores of the second tile already belong to another piece: its Q replaces the first piece's
+  if (nxt.piece >= 0 && nxt.piece != cur.piece) load_q(nxt.piece);
+
+  // One iteration; PAR = buffer of tile j (K(j+1) sits in the other K buffer).
+  auto tile_step = [&](auto PAR) __attribute__((always_inline)) {
+    constexpr int par = decltype(PAR)::value;
+    const char* tV = sV + par * TILE_BYTES;
+    const char* tKn = sK + (par ^ 1) * TILE_BYTES;
+    floatx16 c0 = sn0, c1 = sn1;  // S(j)
+
+    // everything fetched so far has landed (tile copies, a new piece's Q, a finished piece's stores);
+    // after the barrier nobody still reads what comes next
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
+
+    if constexpr (!BOUNDED) {
+      const float mx_s = mx * c;
+      if (__any(mx_s > m_run + RESCALE_SLACK)) {
+        const float m_new = fmaxf(m_run, mx_s);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+        m_run = m_new;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- stage A: S(j+1) = K(j+1) Q^T, the copies of K(j+2) and V(j+1), the softmax of S(j) -------
+    uint32_t pk0[8], pk1[8];
+    float lsum = 0.f;
+    float tf[2][2], te[2][2];
+    auto expo_slot = [&](int n) __attribute__((always_inline)) {
+      if (n >= 2 && n < 18) {
+        const int j = n - 2;
+        lsum += te[j & 1][0] + te[j & 1][1];
+        (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
+      }
+      if (n >= 1 && n < 17) {
+        const int j = n - 1;
+        te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
+        te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
+      }
+      if (n < 16) {
+        const floatx16& cs = n < 8 ? c0 : c1;
+        tf[n & 1][0] = __builtin_fmaf(cs[2 * (n & 7)], c, -m_run);
+        tf[n & 1][1] = __builtin_fmaf(cs[2 * (n & 7) + 1], c, -m_run);
+      }
+    };
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
+      else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
+      if (g < IPW) dma_k1(par, nx2.n0, g);
+      else if (g < 2 * IPW) dma_v1(par ^ 1, nxt.n0, g - IPW);
+      f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
+      expo_slot(g);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      if (g & 1) sn1 = T::mfma32(f[g], qf[4 + (g >> 1)], sn1);
+      else sn0 = T::mfma32(f[g], qf[4 + (g >> 1)], sn0);
+      f[g] = read_vt(tV, 0, g >> 2, g & 3);
+      if (g < 4) expo_slot(8 + g);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    {
+      const int nv1 = valid_keys(nxt.n0);
+      if (nv1 < BN) mask_tail(sn0, sn1, nv1);  // ragged or absent tile j+1
+    }
+    // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
+    if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- stage B: O^T += V(j)^T P(j)^T, the rest of the softmax, the row maximum of S(j+1) ----------
+    float mxa = fmaxf(sn0[0], sn0[1]), mxb = fmaxf(sn1[0], sn1[1]);
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int g = cc * 4 + db;
+        o[db] = T::mfma32(f[g], bfrag, o[db]);
+        f[g] = read_vt(tV, 1, cc, db);
+        if (g < 6) expo_slot(12 + g);
+        if constexpr (!BOUNDED) {
+          if (g < 4) {
+          } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
+          else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
+      vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int g = cc * 4 + db;
+        o[db] = T::mfma32(f[g], bfrag, o[db]);
+        if constexpr (!BOUNDED) {
+          if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    l_run += lsum;
+    if constexpr (!BOUNDED) mx = across(fmaxf(mxa, mxb));
+
+    if (cur.flags & LAST) finish_item(cur);
+
+    // slide the tile window and point the descriptors at what the next iteration copies (this iteration's
+    // copies are all issued); done here, under the last MFMAs, and not behind the next barrier, where every
+    // wavefront of the workgroup would wait for it
+    cur = nxt;
+    nxt = nx2;
+    pull(nx2);
+    aim_k(nx2);
+    aim_v(nxt);
+  };
+
+  aim_k(nx2);
+  aim_v(nxt);
+  while (cur.piece >= 0) {
+    tile_step(std::integral_constant<int, 0>{});
+    if (cur.piece < 0) break;
+    tile_step(std::integral_constant<int, 1>{});
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the wavefront ends
+}
+
+// Folds the partial results of the pieces that attn_fwd_d128_stream_kernel computed in shares (StreamPlan):
+// the log-sum-exp merge of torch's _SDPAMerger over all shares of a piece at once, plus the running pair of a
+// ring accumulation.  16 workgroups per tail piece, 16 query rows each; one thread = 8 consecutive output elements.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_stream_merge_kernel(const AttnParams p) {
+  if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  const StreamPlan& sp = p.st;
+  const int tp = blockIdx.x >> 4;  // tail piece
+  const int local = ((blockIdx.x & 15) << 4) + (threadIdx.x >> 4);
+  const int c8 = (threadIdx.x & 15) * 8;
+  const int tail0 = sp.R * sp.G;
+  const int64_t Ttail = (int64_t)(sp.n_pieces - tail0) * sp.L;
+  // workgroup whose range holds tail step t: the largest g with g * Ttail / Gt <= t
+  auto slot = [&](int64_t t) { return (int)(((t + 1) * sp.Gt + Ttail - 1) / Ttail) - 1; };
+  const int g_first = slot((int64_t)tp * sp.L), g_last = slot((int64_t)(tp + 1) * sp.L - 1);
+  if (g_first == g_last) return;  // computed whole by one workgroup, which stored it itself
+  const int piece = tail0 + tp;
+  const int bh = piece / p.n_qtiles, qt = piece - bh * p.n_qtiles;
+  const int head = bh % p.H, batch = bh / p.H;
+  const int qrow = qt * 256 + local;
+  if (qrow >= p.Sq) return;
+  const int64_t ridx = ((int64_t)batch * p.H + head) * p.Sq + qrow;
+  auto part_row = [&](int g) { return (int64_t)(2 * g + (g == g_first ? 1 : 0)) * 256 + local; };
+  const float old = (p.acc_out != nullptr && !p.acc_first) ? p.acc_lse[ridx] : -INFINITY;
+  float m = old;
+  for (int g = g_first; g <= g_last; ++g) m = fmaxf(m, p.ws_lse[part_row(g)]);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+  if (old > -INFINITY) {
+    const float w = __expf(old - m);
+    const float4 a = *(const float4*)(p.acc_out + ridx * 128 + c8);
+    const float4 b = *(const float4*)(p.acc_out + ridx * 128 + c8 + 4);
+    den = w;
+    acc[0] = w * a.x; acc[1] = w * a.y; acc[2] = w * a.z; acc[3] = w * a.w;
+    acc[4] = w * b.x; acc[5] = w * b.y; acc[6] = w * b.z; acc[7] = w * b.w;
+  }
+  if (m > -INFINITY) {
+    for (int g = g_first; g <= g_last; ++g) {
+      const int64_t wrow = part_row(g);
+      const float w = __expf(p.ws_lse[wrow] - m);  // an empty share has LSE -inf: weight 0
+      const float4 a = *(const float4*)(p.ws_out + wrow * 128 + c8);
+      const float4 b = *(const float4*)(p.ws_out + wrow * 128 + c8 + 4);
+      den += w;
+      acc[0] += w * a.x; acc[1] += w * a.y; acc[2] += w * a.z; acc[3] += w * a.w;
+      acc[4] += w * b.x; acc[5] += w * b.y; acc[6] += w * b.z; acc[7] += w * b.w;
+    }
+  }
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  if (p.out != nullptr) {
+    u32x4 w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = T::pack2(acc[2 * i] * inv, acc[2 * i + 1] * inv);
+    uint16_t* op = (uint16_t*)p.out + batch * p.os_b + head * p.os_h + (int64_t)qrow * p.os_s + c8;
+    *(u32x4*)op = w;
+  } else {
+    float* ap = p.acc_out + ridx * 128 + c8;
+    *(float4*)ap = float4{acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+    *(float4*)(ap + 4) = float4{acc[4] * inv, acc[5] * inv, acc[6] * inv, acc[7] * inv};
+  }
+  float* lse_dst = p.acc_out != nullptr ? p.acc_lse : p.lse;
+  if (lse_dst != nullptr && c8 == 0) lse_dst[ridx] = den > 0.f ? m + __logf(den) : -INFINITY;
+}
+
 // Folds the split_s partial results of each split query tile into out and lse: the log-sum-exp
 // merge of torch's _SDPAMerger (used by src/para_attn/sparse_attn.py:174-189) over all pieces at
 // once.  One thread = 8 consecutive output elements of one query row; 16 rows per workgroup.
@@ -1826,16 +2449,18 @@ __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int
 // ---------------------------------------------------------------------------------------------
 constexpr int BOUND_G = 1024;                                   // blocks per tensor
 constexpr size_t BOUND_WS_BYTES = (2 * BOUND_G + 64) * 4;       // partial maxima + the flag word (+ padding)
+// with the keys in n segments: one set of partial maxima per segment, then the flag word
+static inline size_t bound_ws_bytes(int nseg) { return ((size_t)2 * BOUND_G * (nseg < 1 ? 1 : nseg) + 64) * 4; }
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnParams p, float* part) {
+__global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnParams p, float* part, const void* keys, int n_keys) {
   constexpr int LPR = D / 8;       // lanes per row: 8 elements each
   constexpr int RPB = 256 / LPR;   // rows per block and step
   const bool is_k = blockIdx.x >= BOUND_G;
   const int blk = is_k ? blockIdx.x - BOUND_G : blockIdx.x;
-  const uint16_t* base = (const uint16_t*)(is_k ? p.k : p.q);
+  const uint16_t* base = (const uint16_t*)(is_k ? keys : p.q);  // keys: p.k, or one segment of the keys
   const int64_t sb = is_k ? p.ks_b : p.qs_b, sh = is_k ? p.ks_h : p.qs_h, ss = is_k ? p.ks_s : p.qs_s;
-  const int S = is_k ? p.Skv : p.Sq;
+  const int S = is_k ? n_keys : p.Sq;
   const int64_t rows = (int64_t)p.B * p.H * S;
   const int sub = threadIdx.x % LPR;
   float best = 0.f;
@@ -1867,12 +2492,13 @@ __global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnPara
   if (threadIdx.x == 0) part[blockIdx.x] = sm[0];
 }
 
-__global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part, float scale_log2, float limit, int* flag) {
+__global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part, int nparts, float scale_log2, float limit, int* flag) {
   __shared__ float sq[256], sk[256];
   float mq = 0.f, mk = 0.f;
-  for (int i = threadIdx.x; i < BOUND_G; i += 256) {
-    mq = fmaxf(mq, part[i]);
-    mk = fmaxf(mk, part[BOUND_G + i]);
+  for (int i = threadIdx.x; i < BOUND_G * nparts; i += 256) {  // nparts sets of (BOUND_G for Q, BOUND_G for a key segment)
+    const int set = i / BOUND_G, e = i - set * BOUND_G;
+    mq = fmaxf(mq, part[2 * BOUND_G * set + e]);
+    mk = fmaxf(mk, part[2 * BOUND_G * set + BOUND_G + e]);
   }
   sq[threadIdx.x] = mq;
   sk[threadIdx.x] = mk;
@@ -1975,6 +2601,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.bound_flag = nullptr;
   p.mask = nullptr; p.ms_b = p.ms_h = p.ms_q = p.ms_k = 0;
   p.gate = nullptr; p.gate_want = 0;
+  p.st = StreamPlan{};
 }
 
 template <typename T, int D, bool SPARSE>
@@ -2099,8 +2726,10 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
 //   PARAATTN_NO_SPLIT=1      "no_split"      no key-split tail
 //   PARAATTN_NO_XCD_ORDER=1  "no_xcd_order"  block-sparse workgroups in plain order
 //   PARAATTN_BOUND=0|1       "bound"         never / always compute the score bound (-1 = by size)
+//   PARAATTN_STREAM=0|1      "stream"        never / wherever possible the resident-workgroup kernel (-1 = by shape)
+//   PARAATTN_STREAM_EVEN=0|1 "stream_even"   its tail cut into shares that begin at the same keys / into equal ranges (-1 = by size)
 struct Tuning {
-  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound;
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even;
 };
 static Tuning& tuning() {
   static Tuning t;
@@ -2115,6 +2744,10 @@ static Tuning& tuning() {
     t.forced_bm = num("PARAATTN_BM", 0);
     const int b = num("PARAATTN_BOUND", -1);
     t.bound = b == 0 || b == 1 ? b : -1;
+    const int st = num("PARAATTN_STREAM", -1);
+    t.stream = st == 0 || st == 1 ? st : -1;
+    const int se = num("PARAATTN_STREAM_EVEN", -1);
+    t.stream_even = se == 0 || se == 1 ? se : -1;
     return true;
   }();
   (void)init;
@@ -2131,6 +2764,8 @@ extern "C" int pa_set_tuning(const char* name, int value) {
     if (value != 0 && value != 128 && value != 256) PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: bm must be 0, 128 or 256");
     t.forced_bm = value;
   } else if (!strcmp(name, "bound")) t.bound = value == 0 || value == 1 ? value : -1;
+  else if (!strcmp(name, "stream")) t.stream = value == 0 || value == 1 ? value : -1;
+  else if (!strcmp(name, "stream_even")) t.stream_even = value == 0 || value == 1 ? value : -1;
   else PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: unknown knob '%s'", name);
   return PA_OK;
 }
@@ -2221,13 +2856,154 @@ static bool bound_wanted(int B, int H, int Sq, int Skv, int D) {
   return (double)Sq * Skv >= 6144.0 * ((double)Sq + Skv) && 4.0 * B * H * (double)Sq * (double)Skv * D >= 1.0e12;
 }
 
+// The keys and values of a dense launch in several segments of equal length (the blocks of a ring sweep).
+struct KeySegs {
+  int n, len;
+  const void* const* k;
+  const void* const* v;
+};
+
+// Plan for attn_fwd_d128_stream_kernel (see StreamPlan).  Returns false where that kernel does not apply or is
+// not expected to pay; otherwise fills p.st, p.bm, p.n_qtiles, and *ws_need with the bytes of workspace its
+// partial results take (0: no piece is cut).  `sizing`: report the plan that a sufficient workspace would get.
+static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_avail, bool sizing, size_t* ws_need) {
+  *ws_need = 0;
+  const bool multi = segs != nullptr;
+  const int want = tuning().stream;
+  if (want == 0 || (multi && want < 0)) return false;  // key segments: attn_fwd_d128_pipe_kernel walks them too, faster on long sweeps
+  if (D != 128 || p.causal || p.kv_len != nullptr || tuning().no_pipe) return false;
+  const int cus = device_cus();
+  if (cus <= 0) return false;
+  const int seg_len = multi ? segs->len : p.Skv, nseg = multi ? segs->n : 1;
+  if (seg_len <= 0 || nseg <= 0 || nseg > MAX_KEY_SEGS || p.Sq <= 0) return false;
+  if ((uint64_t)(seg_len - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB || (uint64_t)(seg_len - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB)
+    return false;
+  const int tps = (seg_len + BN - 1) / BN;
+  const int64_t L64 = (int64_t)nseg * tps;
+  const int nqt = (p.Sq + 255) / 256;
+  const int64_t P64 = (int64_t)p.B * p.H * nqt;
+  if (L64 > 0x3fffffff || P64 > 0x3fffffff) return false;
+  const int L = (int)L64, P = (int)P64;
+  // Where it pays (measured).  A workgroup per piece spends about 11 key tiles' time on what is not the key
+  // sweep, and a partly filled last round idles the chip; resident workgroups hide the first and cut the second
+  // finely.  But their loop carries more scalar bookkeeping per key tile (15 % more clocks per tile, which the
+  // power-limited chip answers with 8 % more clock: 5-7 % slower per tile), so they win where pieces are short
+  // (up to 16 key tiles: cross-attention to a text prompt) or the launch has fewer than two rounds of pieces and
+  // the last one is partly filled (image models: FLUX has 1.7), and lose on long launches of many rounds.
+  if (!multi && want < 0) {
+    const int rounds = P / cus, left = P % cus;
+    const bool short_pieces = L <= 16 && P >= 2 * cus;
+    const bool ragged_rounds = rounds <= 1 && left > 0 && (int64_t)P * L >= 16 * (int64_t)cus;
+    if (!short_pieces && !ragged_rounds) return false;
+  }
+  StreamPlan& st = p.st;
+  st.G = cus;
+  st.R = P / st.G;
+  st.L = L;
+  st.n_pieces = P;
+  st.nseg = nseg;
+  st.seg_len = seg_len;
+  st.tps = tps;
+  for (int i = 0; i < nseg; ++i) {
+    st.kseg[i] = multi ? segs->k[i] : p.k;
+    st.vseg[i] = multi ? segs->v[i] : p.v;
+  }
+  const int p_tail = P - st.R * st.G;
+  st.Gt = 0;
+  if (p_tail > 0) {
+    const int64_t t_tail = (int64_t)p_tail * L;
+    // K and V of one head: where the L2s hold that (4 MB each), workgroups need not sweep the keys in step
+    const double head_bytes = (double)L * BN * ((double)p.ks_s + (double)p.vs_s) * 2.0;
+    const int ev = tuning().stream_even;
+    const bool even = ev >= 0 ? ev == 1 : head_bytes <= 6.0e6;
+    int gt;
+    if (even) {
+      const int64_t by_size = t_tail / 8;  // at least 8 key tiles per workgroup
+      gt = (int)(by_size < st.G ? (by_size < 1 ? 1 : by_size) : st.G);
+    } else {
+      int sh = st.G / p_tail;
+      if (sh > 8) sh = 8;
+      if (sh > L / 16) sh = L / 16;
+      if (sh < 1) sh = 1;
+      gt = p_tail * sh;
+    }
+    if (tuning().no_split) gt = p_tail;
+    size_t need = gt != p_tail ? (size_t)2 * gt * 256 * (128 + 1) * sizeof(float) : 0;
+    if (need > ws_avail && !sizing) {  // whole pieces only
+      gt = p_tail;
+      need = 0;
+    }
+    st.Gt = gt;
+    *ws_need = need;
+  }
+  p.pipe = 1;
+  p.bm = 256;
+  p.n_qtiles = nqt;
+  p.split_s = 0;
+  return true;
+}
+
+template <typename T>
+static int launch_stream(const AttnParams& p, hipStream_t stream) {
+  if (p.out == nullptr && p.acc_out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
+  const size_t smem = 4 * TILE_BYTES;
+  static bool attr_done[PA_MAX_DEVICES][2] = {};  // benign race: the call is idempotent
+  const int dev = current_device();
+  for (int b = 0; b < 2; ++b) {
+    if (b == 1 && p.bound_flag == nullptr) break;
+    if (dev >= 0 && attr_done[dev][b]) continue;
+    const void* fn = b ? (const void*)attn_fwd_d128_stream_kernel<T, true> : (const void*)attn_fwd_d128_stream_kernel<T, false>;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    if (dev >= 0) attr_done[dev][b] = true;
+  }
+  if (p.bound_flag != nullptr) {  // one of the two variants leaves at once
+    hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, true>), dim3((unsigned)p.st.G), dim3(512), smem, stream, p);
+    PA_CHECK_LAUNCH("attention kernel (resident workgroups, bounded scores)");
+  }
+  hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, false>), dim3((unsigned)p.st.G), dim3(512), smem, stream, p);
+  PA_CHECK_LAUNCH("attention kernel (resident workgroups)");
+  const int p_tail = p.st.n_pieces - p.st.R * p.st.G;
+  if (p_tail > 0 && p.st.Gt != p_tail) {
+    hipLaunchKernelGGL((attn_stream_merge_kernel<T>), dim3((unsigned)p_tail * 16), dim3(256), 0, stream, p);
+    PA_CHECK_LAUNCH("attention share merge kernel");
+  }
+  return PA_OK;
+}
+
+// Launches the two small kernels that bound the scores (see score_bound_partial_kernel) into `ws` and returns the flag's address.
+static int launch_bound(const AttnParams& p, int dtype, int D, const KeySegs* segs, void* ws, hipStream_t st, const int** flag_out) {
+  float* part = (float*)ws;
+  const int nseg = segs ? segs->n : 1;
+  int* flag = (int*)(part + (size_t)2 * BOUND_G * nseg);
+  const float limit = dtype == PA_DTYPE_BF16 ? 60.f : 14.f;
+  for (int i = 0; i < nseg; ++i) {
+    const void* keys = segs ? segs->k[i] : p.k;
+    const int n_keys = segs ? segs->len : p.Skv;
+    float* dst = part + (size_t)2 * BOUND_G * i;
+    if (dtype == PA_DTYPE_BF16 && D == 128)
+      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 128>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+    else if (dtype == PA_DTYPE_BF16)
+      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 64>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+    else if (D == 128)
+      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 128>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+    else
+      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 64>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+    PA_CHECK_LAUNCH("score bound kernel");
+  }
+  hipLaunchKernelGGL(score_bound_flag_kernel, dim3(1), dim3(256), 0, st, (const float*)part, nseg, p.scale_log2, limit, flag);
+  PA_CHECK_LAUNCH("score bound flag kernel");
+  *flag_out = flag;
+  return PA_OK;
+}
+
 static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out, float* lse,
                           int dtype, int B, int H, int Sq, int Skv, int D,
                           const int64_t q_strides[3], const int64_t k_strides[3],
                           const int64_t v_strides[3], const int64_t out_strides[3], float scale,
                           const int32_t* kv_len, int is_causal, void* workspace, size_t workspace_bytes,
                           void* stream, float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0,
-                          const int* gate = nullptr, int gate_want = 0) {
+                          const int* gate = nullptr, int gate_want = 0, const KeySegs* segs = nullptr) {
   const int64_t zero3[3] = {0, 0, 0};
   const bool accumulate = acc_out != nullptr;
   if (accumulate) {
@@ -2245,35 +3021,48 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   p.causal = is_causal != 0;
   p.gate = gate;
   p.gate_want = gate_want;
-  // a workspace that has room for them beside the key split's partials starts with BOUND_WS_BYTES for the score bound
   const size_t ws_avail = workspace ? workspace_bytes : 0;
   char* ws_base = (char*)workspace;
-  choose_kernel(p, D, 256, true, ws_avail, nullptr);
-  const size_t split_bytes = p.split_s > 1 ? (size_t)p.split_tiles * p.split_s * p.bm * (128 + 1) * sizeof(float) : 0;
-  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && (D == 64 || p.bm == 256) && ws_avail >= split_bytes + BOUND_WS_BYTES) {
-    ws_base += BOUND_WS_BYTES;
-    float* part = (float*)workspace;
-    int* flag = (int*)(part + 2 * BOUND_G);
-    const float limit = dtype == PA_DTYPE_BF16 ? 60.f : 14.f;
-    if (dtype == PA_DTYPE_BF16 && D == 128)
-      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 128>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
-    else if (dtype == PA_DTYPE_BF16)
-      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 64>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
-    else if (D == 128)
-      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 128>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
-    else
-      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 64>), dim3(2 * BOUND_G), dim3(256), 0, (hipStream_t)stream, p, part);
-    PA_CHECK_LAUNCH("score bound kernel");
-    hipLaunchKernelGGL(score_bound_flag_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)part, p.scale_log2, limit, flag);
-    PA_CHECK_LAUNCH("score bound flag kernel");
-    p.bound_flag = flag;
+  const int nseg = segs ? segs->n : 1;
+  // the workspace starts with the score bound's words where there is room for them beside the partial results
+  const size_t bound_bytes = bound_ws_bytes(nseg);
+  const bool want_bound = bound_wanted(B, H, Sq, Skv, D);
+  size_t stream_bytes = 0;
+  bool streamed = plan_stream(p, D, segs, ws_avail > bound_bytes && want_bound ? ws_avail - bound_bytes : ws_avail, false, &stream_bytes);
+  if (!streamed) choose_kernel(p, D, 256, true, ws_avail, nullptr);
+  if (segs && !streamed) {
+    if (D != 128 || !p.pipe || p.causal || kv_len != nullptr || segs->n > MAX_KEY_SEGS ||
+        (uint64_t)(segs->len - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB || (uint64_t)(segs->len - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB)
+      PA_FAIL(PA_ERR_UNSUPPORTED, "a sweep over key segments needs head_dim 128, at most %d segments, all keys together below 4 GiB per head, no causal mask", MAX_KEY_SEGS);
+    if (p.split_s > segs->n) p.split_s = 0;  // a key share is a run of whole segments
+    p.st.nseg = segs->n;
+    p.st.seg_len = segs->len;
+    for (int i = 0; i < segs->n; ++i) {
+      p.st.kseg[i] = segs->k[i];
+      p.st.vseg[i] = segs->v[i];
+    }
+  }
+  const size_t split_bytes = streamed ? stream_bytes
+                             : p.split_s > 1 ? (size_t)p.split_tiles * p.split_s * p.bm * (128 + 1) * sizeof(float) : 0;
+  if (want_bound && p.pipe && (D == 64 || p.bm == 256) && ws_avail >= split_bytes + bound_bytes) {
+    ws_base += bound_bytes;
+    rc = launch_bound(p, dtype, D, segs, workspace, (hipStream_t)stream, &p.bound_flag);
+    if (rc) return rc;
   }
   if (accumulate) {
     if (p.causal) PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation is not causal");
-    if (!p.pipe || D != 128)  // only the head_dim-128 pipelined kernel has the folding epilogue
+    if (!p.pipe || D != 128)  // only the head_dim-128 pipelined kernels have the folding epilogue
       PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation needs head_dim 128 and K/V below 4 GiB per head; run pa_attn_fwd_lse and pa_merge_lse");
     p.acc_out = acc_out; p.acc_lse = acc_lse; p.acc_first = acc_first != 0;
     p.lse = nullptr;
+  }
+  if (streamed) {
+    if (stream_bytes > 0) {
+      p.ws_out = (float*)ws_base;
+      p.ws_lse = p.ws_out + (size_t)2 * p.st.Gt * 256 * 128;
+    }
+    if (B == 0 || H == 0 || Sq == 0) return PA_OK;
+    return dtype == PA_DTYPE_BF16 ? launch_stream<BF16>(p, (hipStream_t)stream) : launch_stream<F16>(p, (hipStream_t)stream);
   }
   if (p.split_s > 1) {
     p.ws_out = (float*)ws_base;
@@ -2314,6 +3103,43 @@ extern "C" int pa_attn_fwd_accumulate(const void* q, const void* k, const void* 
                         out_strides, scale, kv_len, 0, workspace, workspace_bytes, stream, acc_out, acc_lse, first);
 }
 
+extern "C" int pa_attn_fwd_sweep(const void* q, const void* const* k_blocks, const void* const* v_blocks, int n_blocks,
+                                 int block_len, void* out, float* lse, int dtype, int B, int H, int Sq, int D,
+                                 const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                                 const int64_t out_strides[3], float scale, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+  if (!k_blocks || !v_blocks) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+  if (n_blocks <= 0 || n_blocks > MAX_KEY_SEGS) PA_FAIL(PA_ERR_UNSUPPORTED, "a sweep takes 1 to %d key/value blocks (got %d)", MAX_KEY_SEGS, n_blocks);
+  if (block_len <= 0) PA_FAIL(PA_ERR_INVALID, "key/value blocks must not be empty");
+  if ((int64_t)n_blocks * block_len > 0x7fffffffLL) PA_FAIL(PA_ERR_UNSUPPORTED, "too many keys");
+  for (int i = 0; i < n_blocks; ++i) {
+    if (!k_blocks[i] || !v_blocks[i]) PA_FAIL(PA_ERR_INVALID, "null pointer argument");
+    if (((uintptr_t)k_blocks[i]) % 16 || ((uintptr_t)v_blocks[i]) % 16) PA_FAIL(PA_ERR_UNSUPPORTED, "key/value block pointer not 16-byte aligned");
+  }
+  if (D != 128) PA_FAIL(PA_ERR_UNSUPPORTED, "a sweep over key/value blocks needs head_dim 128 (got %d)", D);
+  const KeySegs segs = {n_blocks, block_len, k_blocks, v_blocks};
+  return attn_fwd_dense(q, k_blocks[0], v_blocks[0], out, lse, dtype, B, H, Sq, n_blocks * block_len, D, q_strides,
+                        k_strides, v_strides, out_strides, scale, nullptr, 0, workspace, workspace_bytes, stream,
+                        nullptr, nullptr, 0, nullptr, 0, &segs);
+}
+
+extern "C" size_t pa_attn_fwd_sweep_workspace_bytes(int B, int H, int Sq, int n_blocks, int block_len, int D,
+                                                    const int64_t k_strides[3], const int64_t v_strides[3]) {
+  if (B <= 0 || H <= 0 || Sq <= 0 || n_blocks <= 0 || n_blocks > MAX_KEY_SEGS || block_len <= 0 || D != 128 || !k_strides || !v_strides) return 0;
+  AttnParams p;
+  const int64_t zero[3] = {0, 0, 0};
+  fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, n_blocks * block_len, zero, k_strides, v_strides, zero, 1.f);
+  const void* none[MAX_KEY_SEGS] = {};
+  const KeySegs segs = {n_blocks, block_len, none, none};
+  size_t need = 0;
+  if (!plan_stream(p, D, &segs, 0, true, &need)) {
+    choose_kernel(p, D, 256, true, 0, &need);
+    if (!p.pipe) return 0;
+  }
+  if (bound_wanted(B, H, Sq, n_blocks * block_len, D) && p.bm == 256) need += bound_ws_bytes(n_blocks);
+  return need;
+}
+
 extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
                                               const int64_t k_strides[3], const int64_t v_strides[3]) {
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || (D != 128 && D != 64) || !k_strides || !v_strides) return 0;
@@ -2321,7 +3147,7 @@ extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int
   const int64_t zero[3] = {0, 0, 0};
   fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
   size_t need = 0;
-  choose_kernel(p, D, 256, true, 0, &need);
+  if (!plan_stream(p, D, nullptr, 0, true, &need)) choose_kernel(p, D, 256, true, 0, &need);
   if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && (D == 64 || p.bm == 256)) need += BOUND_WS_BYTES;
   return need;
 }

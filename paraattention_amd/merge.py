@@ -58,14 +58,28 @@ class SDPAMerger:
         return out, self._lse.reshape(self._lse_shape)
 
 
+def _sweepable(query, key_blocks, value_blocks):
+    """Whether ``para_attn::attention_forward_sweep`` takes these blocks (head_dim 128, at most 16 blocks of one
+    shape, dtype and device, each below 4 GiB per head)."""
+    k0 = key_blocks[0]
+    if query.shape[-1] != 128 or not 1 < len(key_blocks) <= 16 or k0.shape[2] == 0:
+        return False
+    if k0.shape[2] * max(k0.stride(2), value_blocks[0].stride(2), 128) * 2 >= (1 << 32) - 8192:
+        return False
+    return all(t.shape == k0.shape and t.dtype == query.dtype and t.device == query.device for t in list(key_blocks) + list(value_blocks))
+
+
 def ring_sweep(query, key_blocks, value_blocks, *, scale=None, fused=None):
     """One rank's ring-attention pass: ``query`` against successive key/value blocks.
 
-    Equals one SDPA of ``query`` over the concatenation of all blocks.  The last
-    merge writes the activation dtype directly, so no separate cast pass runs.
-    ``fused`` (default: when the accumulator is fp32, head_dim is 128 and there is
-    more than one block) folds each block's result into the accumulator inside
-    the attention kernel; ``fused=False`` runs attention and merge as two launches.
+    Equals one SDPA of ``query`` over the concatenation of all blocks.  ``fused``:
+      "sweep"  one launch walks all blocks and carries the softmax state across them in registers (the default
+               where the blocks allow it: they are all resident on this GPU, which is what a one-rank sweep is);
+      True     one launch per block, each folding its result into an fp32 running pair inside the attention
+               kernel (what a rank of a real ring does as blocks arrive; the default otherwise when the
+               accumulator is fp32 and head_dim is 128);
+      False    attention and merge as two launches per block.
+    The last step writes the activation dtype directly, so no separate cast pass runs.
     Returns (out in query.dtype, fp32 lse [B,H,Sq]).
     """
     assert len(key_blocks) == len(value_blocks) and len(key_blocks) > 0
@@ -73,7 +87,9 @@ def ring_sweep(query, key_blocks, value_blocks, *, scale=None, fused=None):
     acc_dtype = torch.float32 if convert else query.dtype
     n = len(key_blocks)
     if fused is None:
-        fused = convert and n > 1 and query.shape[-1] == 128
+        fused = "sweep" if _sweepable(query, key_blocks, value_blocks) else (convert and n > 1 and query.shape[-1] == 128)
+    if fused == "sweep":
+        return ops.attention_forward_sweep(query, list(key_blocks), list(value_blocks), scale=scale)
     if fused:
         # attention and merge in one launch per block: the blocks' own outputs never exist
         B, H, Sq, D = query.shape

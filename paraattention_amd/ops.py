@@ -16,6 +16,7 @@ Ops the reference has no name for, because there the arithmetic is a chain of
 torch elementwise calls:
   merge_attention_lse / merge_attention_lse_   (torch _SDPAMerger._merge_one)
   attention_forward_accumulate_ / _final       (attention + merge step in one launch)
+  attention_forward_sweep                      (a whole ring sweep over resident key/value blocks in one launch)
   attention_forward_block_sparse               (sparse_attn.py:74-278)
   block_sparse_key_runs, attention_forward_block_sparse_runs  (the same with the mask's run scan done once)
   fbcache_residual_diff                        (first_block_cache/utils.py:228-233)
@@ -39,6 +40,10 @@ def _stream_ptr(device):
 
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
 
 
 def _kernel_ready(t):
@@ -401,6 +406,58 @@ def _(acc_out, acc_lse, query, key, value, *, scale=None):
     return query.new_empty(query.shape)
 
 
+@torch.library.custom_op("para_attn::attention_forward_sweep", mutates_args=(), device_types=("cuda",))
+def attention_forward_sweep(
+    query: torch.Tensor,
+    key_blocks: List[torch.Tensor],
+    value_blocks: List[torch.Tensor],
+    *,
+    scale: Optional[float] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """A whole same-GPU ring sweep in one launch: SDPA of ``query`` over the concatenation of the key/value
+    blocks, which stay where they are (what the loop of src/para_attn/para_attn_interface.py:164-197 computes with
+    one attention call and one merge per block).  Returns (out in query's dtype, fp32 LSE [B,H,Sq]).
+    Blocks must share shape, dtype and strides; head_dim 128; at most 16 blocks (NotImplementedError otherwise)."""
+    n = len(key_blocks)
+    if n == 0 or len(value_blocks) != n:
+        raise ValueError("key_blocks and value_blocks must be non-empty lists of equal length")
+    _check_sdpa_args(query, key_blocks[0], value_blocks[0], 0.0, False)
+    B, H, Sq, D = query.shape
+    ks = [_kernel_ready(t) for t in key_blocks]
+    vs = [_kernel_ready(t) for t in value_blocks]
+    for t in ks + vs:
+        if t.shape != ks[0].shape or t.dtype != query.dtype or t.device != query.device:
+            raise ValueError("all key/value blocks must share the first key block's shape, and the query's dtype and device")
+    if any(t.stride() != ks[0].stride() for t in ks) or any(t.stride() != vs[0].stride() for t in vs):
+        ks = [t.contiguous() for t in ks]
+        vs = [t.contiguous() for t in vs]
+    blk = ks[0].shape[2]
+    q = _kernel_ready(query)
+    out = torch.empty_like(q)
+    if out.stride(-1) != 1:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        kst, vst = _lib.strides3(ks[0]), _lib.strides3(vs[0])
+        ws_bytes = lib.pa_attn_fwd_sweep_workspace_bytes(B, H, Sq, n, blk, D, kst, vst)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+        rc = lib.pa_attn_fwd_sweep(
+            _ptr(q), _ptr_array(ks), _ptr_array(vs), n, blk, _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, D,
+            _lib.strides3(q), kst, vst, _lib.strides3(out), float(scale), _ptr(ws), ws_bytes, _stream_ptr(q.device),
+        )
+    _lib.check(rc, "pa_attn_fwd_sweep")
+    return out, lse
+
+
+@torch.library.register_fake("para_attn::attention_forward_sweep")
+def _(query, key_blocks, value_blocks, *, scale=None):
+    B, H, Sq, _ = query.shape
+    return query.new_empty(query.shape), query.new_empty((B, H, Sq), dtype=torch.float32)
+
+
 # ---------------------------------------------------------------------------------
 # block-sparse attention
 # ---------------------------------------------------------------------------------
@@ -730,10 +787,6 @@ def _flat_same(tensors, what):
             raise ValueError(f"{what}: tensors must share shape, dtype and device")
         out.append(t if t.is_contiguous() and t.data_ptr() % 16 == 0 else t.contiguous().clone())
     return out
-
-
-def _ptr_array(tensors):
-    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
 
 
 @torch.library.custom_op("para_attn::taylorseer_derivatives", mutates_args=(), device_types=("cuda",))

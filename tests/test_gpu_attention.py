@@ -388,6 +388,49 @@ def test_key_split_tail(cuda, bm, tuning):
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
 
 
+@pytest.mark.parametrize("even", [-1, 0, 1])
+@pytest.mark.parametrize("bound", [0, 1])
+def test_resident_workgroup_kernel(cuda, even, bound, tuning):
+    """The kernel whose workgroups stay resident and walk a list of pieces as one stream of key tiles, forced on
+    for every shape here: fewer pieces than compute units (every piece cut into ranges), a few pieces more than a
+    whole number of rounds (whole pieces, then a tail cut evenly or into shares that begin at the same keys),
+    pieces of one and two key tiles (a new piece's Q and output on every iteration), ragged query and key ends,
+    strided memory, both score-bound variants.  Against the fp64 oracle, and against the kernel with one
+    workgroup per piece."""
+    tuning("stream", 1)
+    tuning("stream_even", even)
+    tuning("bound", bound)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    op = torch.ops.para_attn.attention_forward_with_lse
+    shapes = [(1, 2, 300, 434), (2, 3, 129, 1000), (1, 1, 64, 64), (1, 3, 1000, 77), (2, 2, 700, 128), (1, 5, 2000, 40),
+              (1, 2, (cus // 2 + 5) * 256 - 19, 64 * 40 + 37), (2, 4, (2 * cus // 8 + 3) * 256, 100), (1, 1, (cus + 1) * 256, 64)]
+    for B, H, Sq, Skv in shapes:
+        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=Sq + Skv)
+        qd = q.to(cuda).transpose(1, 2).contiguous().transpose(1, 2)
+        kd, vd = k.to(cuda), v.to(cuda)
+        out, lse = op(qd, kd, vd)
+        rows = torch.arange(Sq) if Sq <= 2000 else torch.cat([torch.arange(0, 300), torch.arange(Sq - 600, Sq)])
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), k.float().numpy(), v.float().numpy())
+        _check(out[:, :, rows.to(cuda)], lse[:, :, rows.to(cuda)], ref_out, ref_lse, f"resident {(B, H, Sq, Skv)} even={even} bound={bound}")
+        tuning("stream", 0)
+        out0, lse0 = op(qd, kd, vd)
+        tuning("stream", 1)
+        assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
+        assert torch.equal(torch.ops.para_attn.attention_forward(qd, kd, vd), out)
+    # the shapes the planner picks it for by itself: FLUX's 1.7 rounds and short cross-attention pieces
+    # (its partial results are what FLUX's workspace is for: the one-workgroup-per-piece plan has no split there)
+    tuning("stream", -1)
+    tuning("stream_even", -1)
+    from paraattention_amd import _lib
+
+    lib = _lib.load()
+    qf = torch.empty(1, 24, 4608, 128, dtype=torch.bfloat16, device=cuda)
+    assert lib.pa_attn_fwd_workspace_bytes(1, 24, 4608, 4608, 128, _lib.strides3(qf), _lib.strides3(qf)) > 0
+    tuning("stream", 0)
+    tuning("bound", 0)
+    assert lib.pa_attn_fwd_workspace_bytes(1, 24, 4608, 4608, 128, _lib.strides3(qf), _lib.strides3(qf)) == 0
+
+
 @pytest.mark.parametrize("D,bm", [(128, "256"), (64, "128"), (64, "256")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_score_bound_variants(cuda, dtype, D, bm, tuning):

@@ -98,7 +98,7 @@ def test_merge_empty_partials(cuda):
     assert torch.equal(out.cpu(), o2.float()) and torch.equal(lse.cpu(), l2)
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["sweep", True, False])
 def test_ring_sweep_equals_full_attention(cuda, fused):
     # the ring-sweep shape in miniature, ragged like 14882 = 116*128 + 34: 8 blocks of 290 keys
     B, H, Sq, D, nblk, blk = 1, 4, 290, 128, 8, 290
@@ -110,6 +110,37 @@ def test_ring_sweep_equals_full_attention(cuda, fused):
     assert out.dtype == torch.bfloat16
     np.testing.assert_allclose(lse.cpu().numpy(), ref_lse, atol=1e-3)
     np.testing.assert_allclose(out.float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_one_launch_sweep(cuda, dtype, tuning):
+    """attention_forward_sweep: blocks at separate addresses walked as one key sequence.  Ragged block length
+    (tiles never straddle blocks), ragged query length, [B,S,H,D] memory, 1 to 16 blocks, more pieces than the
+    chip has compute units and fewer, with and without the score bound; against the fp64 oracle over the
+    concatenated keys and bit for bit against the dense op on the concatenation where both take the same path."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    D = 128
+    for B, H, Sq, blk, n, bound in [(1, 2, 300, 290, 8, -1), (2, 3, 77, 64, 3, -1), (1, 4, 600, 1000, 16, 1), (1, 1, 256, 37, 1, -1),
+                                    (1, 2, (cus // 2 + 3) * 256 - 100, 150, 4, 1)]:
+        tuning("bound", bound)
+        q, k, v = inputs.qkv(B, H, Sq, blk * n, D, seed=blk + n, dtype=dtype)
+        rows = torch.arange(Sq) if Sq <= 1000 else torch.cat([torch.arange(0, 50), torch.arange(Sq - 400, Sq, 3)])
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), k.float().numpy(), v.float().numpy())
+        qd = q.to(cuda).transpose(1, 2).contiguous().transpose(1, 2)
+        kb = [t.contiguous().to(cuda) for t in k.split(blk, 2)]
+        vb = [t.contiguous().to(cuda) for t in v.split(blk, 2)]
+        out, lse = torch.ops.para_attn.attention_forward_sweep(qd, kb, vb)
+        assert out.dtype == dtype and out.stride() == qd.stride() and lse.shape == (B, H, Sq)
+        np.testing.assert_allclose(lse[:, :, rows.to(cuda)].cpu().numpy(), ref_lse, atol=1e-3)
+        np.testing.assert_allclose(out[:, :, rows.to(cuda)].float().cpu().numpy(), ref_out, atol=2e-2, rtol=2e-2)
+        # ring_sweep takes this path by default
+        ro, rl = paraattention_amd.ring_sweep(qd, kb, vb)
+        assert torch.equal(ro, out) and torch.equal(rl, lse)
+    with pytest.raises(NotImplementedError):
+        q64, k64, v64 = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 64))
+        torch.ops.para_attn.attention_forward_sweep(q64, [k64, k64], [v64, v64])
+    with pytest.raises(ValueError):
+        torch.ops.para_attn.attention_forward_sweep(qd, kb, vb[:-1])
 
 
 def test_fused_accumulate_steps(cuda, tuning):
