@@ -171,8 +171,10 @@ def bench_wan(dev, steps=10, warmup=3):
 
 
 def bench_ring(dev, steps=5, warmup=2):
-    """One rank's ring pass: a Q block of 14882 tokens x 24 heads against 8 KV blocks of 14882 keys, the merge
-    folded into the attention kernel; checked against one SDPA over all 119056 keys."""
+    """One rank's ring pass: a Q block of 14882 tokens x 24 heads against 8 KV blocks of 14882 keys; checked against
+    one SDPA over all 119056 keys.  Two ways: all blocks in one launch (the softmax state carried across the blocks
+    in registers: what a sweep over resident blocks is), and one launch per block with the fp32 running pair folded
+    inside the attention kernel (what a rank of a real ring does as blocks arrive)."""
     import torch
 
     import paraattention_amd
@@ -183,19 +185,25 @@ def bench_ring(dev, steps=5, warmup=2):
     kb_cpu = [torch.randn(B, H, S, D, generator=g).bfloat16() for _ in range(nblk)]
     vb_cpu = [torch.randn(B, H, S, D, generator=g).bfloat16() for _ in range(nblk)]
     qd, kb, vb = q.to(dev), [t.to(dev) for t in kb_cpu], [t.to(dev) for t in vb_cpu]
-    last = {}
-
-    def call(i):
-        last["out"], last["lse"] = paraattention_amd.ring_sweep(qd, kb, vb)
-
-    t = _time_calls(call, steps, warmup)
     heads = [0, H - 1]
     k_all = torch.cat([kk[:, heads] for kk in kb_cpu], dim=2)
     v_all = torch.cat([vv[:, heads] for vv in vb_cpu], dim=2)
-    checked = _check_rows(last["out"][:, heads], last["lse"][:, heads], q[:, heads], k_all, v_all, [0, 1], _sample_rows(S), "ring sweep")
     flops = 4.0 * B * H * S * S * nblk * D
-    return _mfma("ring sweep: Q block [1,24,14882,128] bf16 against 8 KV blocks of 14882 keys, fp32 accumulation "
-                 "folded into the attention kernel (one launch per block)", flops, t, launches_per_sweep=nblk, checked=checked)
+    out = {}
+    for key, fused, launches, how in (
+        ("ring_sweep", "sweep", 1, "one launch over all blocks, softmax state carried in registers"),
+        ("ring_sweep_per_block", True, nblk, "one launch per block, fp32 running pair folded inside the attention kernel"),
+    ):
+        last = {}
+
+        def call(i):
+            last["out"], last["lse"] = paraattention_amd.ring_sweep(qd, kb, vb, fused=fused)
+
+        t = _time_calls(call, steps, warmup)
+        checked = _check_rows(last["out"][:, heads], last["lse"][:, heads], q[:, heads], k_all, v_all, [0, 1], _sample_rows(S), key)
+        out[key] = _mfma(f"ring sweep: Q block [1,24,14882,128] bf16 against 8 KV blocks of 14882 keys, {how}", flops, t,
+                         launches_per_sweep=launches, checked=checked)
+    return out
 
 
 def bench_shapes(dev, steps=10, warmup=3):
@@ -436,7 +444,8 @@ def main():
         print(json.dumps(result))
         return
     if not args.no_extras:
-        extras = {"flux_joint_attention": bench_flux(dev), "ring_sweep": bench_ring(dev)}
+        extras = {"flux_joint_attention": bench_flux(dev)}
+        extras.update(bench_ring(dev))
         extras.update(bench_wan(dev))
         extras["block_sparse"] = bench_sparse(dev)
         extras["merge_lse"] = bench_merge(dev)

@@ -59,6 +59,8 @@ PA_API const char* pa_last_error(void);
  *   "bound"        PARAATTN_BOUND=0|1       0 / 1: never / always compute the score bound, -1 = by size
  *   "stream"       PARAATTN_STREAM=0|1      0 / 1: never / wherever possible the kernel with resident workgroups, -1 = by shape
  *   "stream_even"  PARAATTN_STREAM_EVEN=0|1 that kernel's tail cut into shares that begin at the same keys / into equal ranges, -1 = by size
+ *   "sparse_pair"  PARAATTN_SPARSE_PAIR=1   1: pa_attn_fwd_blocksparse with 128-row query blocks puts two adjacent blocks into one
+ *                                           256-row workgroup that walks the union of their key ranges (head_dim 128)
  * Returns PA_ERR_INVALID for an unknown name or value.
  */
 PA_API int pa_set_tuning(const char* name, int value);

@@ -85,6 +85,7 @@ struct AttnParams {
   const int32_t* runs;  // count[Hm*nSeg] then range[Hm*nSeg][cap][2]
   int Hm, nQ, cap;
   int q_lo, q_block;
+  int pair;  // block-sparse: each 256-row workgroup holds two 128-row query blocks and walks the union of their ranges
   int tiles_left, tiles_per_block;
   // dense pipelined kernel only: key-split tail.  Workgroups below split_main own a whole query
   // tile; the last split_tiles query tiles are computed by split_s workgroups each, over
@@ -900,7 +901,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 // workgroups in several key shares (AttnParams::split_*), fold the result into a running
 // (out, lse) pair (acc_*), or apply torch's causal mask (causal).
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool SPARSE, int NW, bool BOUNDED = false>
+template <typename T, bool SPARSE, int NW, bool BOUNDED = false, bool PAIR = false>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
   constexpr int DC = 8, DB = 4;
@@ -1062,16 +1063,32 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   // window of tiles j (being consumed), j+1 and j+2: (first key or OOB, valid keys)
   uint32_t n_cur, n_nxt, n_nx2;
   int v_cur, v_nxt, v_nx2;
+  // PAIR (block-sparse, two adjacent 128-row query blocks per workgroup walking the union of their key ranges):
+  // which of the two blocks keeps tiles j, j+1, j+2 (bit 0: the lower block = wavefronts 0..3, bit 1: the
+  // upper); a range's first key carries the bits in its two low bits (ranges begin at multiples of 4 there).
+  int m_cur = 3, m_nxt = 3, m_nx2 = 3;
+  const int my_bit = wave < NW / 2 ? 1 : 2;
   auto pull = [&](uint32_t& n0, int& nv) {
+    if constexpr (PAIR) {
+      m_cur = m_nxt;
+      m_nxt = m_nx2;
+    }
     if (it.valid()) {
       int a, b;
       it.get(a, b);
+      if constexpr (PAIR) {
+        m_nx2 = a & 3;
+        a &= ~3;
+        const int left = it.end - a;
+        b = left < BN ? left : BN;
+      }
       it.next();
       n0 = (uint32_t)a;
       nv = b;
     } else {
       n0 = OOB;
       nv = 0;
+      if constexpr (PAIR) m_nx2 = 0;
     }
   };
   bool have = false;
@@ -1110,8 +1127,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
   for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
 
   // One iteration; PAR = buffer of tile j (K(j+1) sits in the other K buffer).
-  auto tile_step = [&](auto PAR) {
+  // ACUR / ANXT (PAIR only, else both true): whether this wavefront's query block keeps tile j / tile j+1; what
+  // belongs to a tile it does not keep (scores, softmax, second GEMM) is compiled out of that variant, the copies
+  // and the barrier stay.
+  auto tile_step = [&](auto PAR, auto ACUR, auto ANXT) {
     constexpr int par = decltype(PAR)::value;
+    const bool ac = ACUR, an = ANXT;  // constants unless PAIR
     const char* tV = sV + par * TILE_BYTES;
     const char* tKn = sK + (par ^ 1) * TILE_BYTES;
     floatx16 c0 = sn0, c1 = sn1;  // S(j)
@@ -1121,10 +1142,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     __syncthreads();
 
     // first fragments of K(j+1) on their way while the maximum is settled
+    if (an) {
 #pragma unroll
-    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
+      for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
+    }
 
-    if constexpr (!BOUNDED) {
+    if (!BOUNDED && ac) {
       const float mx_s = mx * c;
       if (__any(mx_s > m_run + RESCALE_SLACK)) {
         const float m_new = fmaxf(m_run, mx_s);
@@ -1176,29 +1199,47 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
       // the two halves of S(j+1) alternate, so that no MFMA waits for the one just issued
-      if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
-      else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
+      if (an) {
+        if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
+        else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
+      }
       if (g < IPW) dma_k1(par, n_nx2, g);                      // K(j+2) takes the buffer K(j) has left
       else if (g < 2 * IPW) dma_v1(par ^ 1, n_nxt, g - IPW);  // V(j+1) takes the buffer V(j-1) has left
-      f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
-      expo_slot(g);
+      if (an) f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
+      if (ac) expo_slot(g);
       __builtin_amdgcn_sched_barrier(0);  // keep the groups in this order
     }
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
-      if (g & 1) sn1 = T::mfma32(f[g], qf[4 + (g >> 1)], sn1);
-      else sn0 = T::mfma32(f[g], qf[4 + (g >> 1)], sn0);
-      f[g] = read_vt(tV, 0, g >> 2, g & 3);  // V(j), keys 0..31, takes the slot over
-      if (g < 4) expo_slot(8 + g);
+      if (an) {
+        if (g & 1) sn1 = T::mfma32(f[g], qf[4 + (g >> 1)], sn1);
+        else sn0 = T::mfma32(f[g], qf[4 + (g >> 1)], sn0);
+      }
+      if (ac) {
+        f[g] = read_vt(tV, 0, g >> 2, g & 3);  // V(j), keys 0..31, takes the slot over
+        if (g < 4) expo_slot(8 + g);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (v_nxt < BN || on_diagonal(n_nxt)) mask_tail(sn0, sn1, v_nxt, n_nxt);  // ragged, absent or diagonal tile j+1
+    if (an) {
+      if (v_nxt < BN || on_diagonal(n_nxt)) mask_tail(sn0, sn1, v_nxt, n_nxt);  // ragged, absent or diagonal tile j+1
+    }
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage B ---------------------------------------------------------------------------------
     if constexpr (NW == 4) __builtin_amdgcn_s_setprio(1);
     __builtin_amdgcn_sched_barrier(0);
     float mxa = fmaxf(sn0[0], sn0[1]), mxb = fmaxf(sn1[0], sn1[1]);
+    if (!ac) {
+      if (!BOUNDED && an) {  // no second GEMM to spread the row maximum of S(j+1) under
+#pragma unroll
+        for (int r = 2; r < 16; ++r) {
+          mxa = fmaxf(mxa, sn0[r]);
+          mxb = fmaxf(mxb, sn1[r]);
+        }
+      }
+    }
+    if (ac)
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
@@ -1209,7 +1250,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         o[db] = T::mfma32(f[g], bfrag, o[db]);
         f[g] = read_vt(tV, 1, cc, db);  // keys 32..63
         if (g < 6) expo_slot(12 + g);
-        if constexpr (!BOUNDED) {
+        if (!BOUNDED && an) {
           if (g < 4) {
           } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
           else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
@@ -1217,6 +1258,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    if (ac)
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
@@ -1225,14 +1267,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       for (int db = 0; db < DB; ++db) {
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
-        if constexpr (!BOUNDED) {
+        if (!BOUNDED && an) {
           if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    l_run += lsum;
-    if constexpr (!BOUNDED) mx = across(fmaxf(mxa, mxb));
+    if (ac) l_run += lsum;
+    if (!BOUNDED && an) mx = across(fmaxf(mxa, mxb));
 
     // slide the tile window
     n_cur = n_nxt;
@@ -1291,10 +1333,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         mx = across(m2);
       }
     }
+    auto step = [&](auto PAR) {
+      constexpr std::true_type yes{};
+      if constexpr (!PAIR) {
+        tile_step(PAR, yes, yes);
+      } else {  // wave-uniform: what this wavefront's query block keeps of tiles j and j+1
+        tile_step(PAR, (m_cur & my_bit) != 0, (m_nxt & my_bit) != 0);
+      }
+    };
     while (have) {
-      tile_step(std::integral_constant<int, 0>{});
+      step(std::integral_constant<int, 0>{});
       if (!have) break;
-      tile_step(std::integral_constant<int, 1>{});
+      step(std::integral_constant<int, 1>{});
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the segment, or the wavefront, ends
   }
@@ -2435,6 +2485,74 @@ __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int
   }
 }
 
+// The same lists for pairs of adjacent query blocks: segment 1 + i covers query blocks 2i and 2i + 1 and walks the
+// union of their kept key blocks.  A range is a run of key blocks kept by the same blocks of the pair; its first
+// key carries which in its two low bits (1: the lower query block, 2: the upper, 3: both), so kv_lo, kv_block
+// and Skv are multiples of 4 here.  Up to nK + 2 ranges per segment.  The dense margins belong to both.
+__global__ __launch_bounds__(64) void build_pair_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK,
+                                                             int Skv, int kv_lo, int kv_block, int cap,
+                                                             int32_t* ws) {
+  const int nseg = nQ / 2 + 2;
+  const int idx = blockIdx.x;  // grid = Hm * nseg
+  const int lane = threadIdx.x;
+  const int hm = idx / nseg;
+  const int seg = idx % nseg;
+  int32_t* cnt = ws + idx;
+  int32_t* rg = ws + (size_t)Hm * nseg + (size_t)idx * cap * 2;
+  if (seg == 0 || seg == nseg - 1) {
+    if (lane == 0) {
+      if (Skv > 0) {
+        rg[0] = 0 | 3;
+        rg[1] = Skv;
+      }
+      *cnt = Skv > 0 ? 1 : 0;
+    }
+    return;
+  }
+  const uint8_t* row_a = mask + ((size_t)hm * nQ + 2 * (seg - 1)) * nK;
+  const uint8_t* row_b = row_a + nK;
+  const int kv_hi = kv_lo + nK * kv_block;
+  int n = 0;
+  int cur_b = -1, cur_e = -1, cur_m = 0;  // open range (lane 0 only)
+  auto flush = [&] {
+    if (cur_e > cur_b) {
+      rg[2 * n] = cur_b | cur_m;
+      rg[2 * n + 1] = cur_e;
+      ++n;
+    }
+  };
+  auto push = [&](int b, int e, int m) {
+    if (e <= b || m == 0) return;
+    if (cur_e == b && cur_m == m) {
+      cur_e = e;
+    } else {
+      flush();
+      cur_b = b;
+      cur_e = e;
+      cur_m = m;
+    }
+  };
+  if (lane == 0) push(0, kv_lo, 3);
+  for (int base = 0; base < nK; base += 64) {
+    const int j = base + lane;
+    const uint64_t in_a = __ballot(j < nK && row_a[j] != 0);
+    const uint64_t in_b = __ballot(j < nK && row_b[j] != 0);
+    if (lane == 0) {
+      const int lim = nK - base < 64 ? nK - base : 64;
+      for (int i = 0; i < lim; ++i) {
+        const int m = (int)((in_a >> i) & 1) | ((int)((in_b >> i) & 1) << 1);
+        const int b = kv_lo + (base + i) * kv_block;
+        push(b, b + kv_block, m);
+      }
+    }
+  }
+  if (lane == 0) {
+    push(kv_hi, Skv, 3);
+    flush();
+    *cnt = n;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Score bound for the dense pipelined kernels.  |q.k| <= |q| |k|, so with Mq = the largest row
 // norm of Q and Mk that of K no score leaves [-Mq Mk scale, Mq Mk scale]; in the log2 domain of the
@@ -2592,7 +2710,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.scale_log2 = scale * LOG2E;
   p.kv_len = nullptr;
   p.runs = nullptr;
-  p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.tiles_left = 0; p.tiles_per_block = 0;
+  p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.pair = 0; p.tiles_left = 0; p.tiles_per_block = 0;
   p.bm = BM; p.pipe = 0;
   p.xcd_chunk = 0;
   p.causal = 0;
@@ -2631,7 +2749,7 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
   // the attribute belongs to the function on one device: remembered per device and kernel variant
   if (p.bound_flag != nullptr && (SPARSE || !(D == 128 ? slot == 2 : slot >= 1)))
     PA_FAIL(PA_ERR_UNSUPPORTED, "score bound reached a kernel that does not read it");
-  static bool attr_done[PA_MAX_DEVICES][5] = {};  // benign race: the call is idempotent
+  static bool attr_done[PA_MAX_DEVICES][6] = {};  // benign race: the call is idempotent
   const int dev = current_device();
   if (dev < 0 || !attr_done[dev][slot]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -2656,6 +2774,19 @@ static int launch_attn(const AttnParams& p, hipStream_t stream) {
       else
         hipLaunchKernelGGL((attn_fwd_d64_pipe_kernel<T, false, 4, true>), dim3((unsigned)nblocks), dim3(256), smem, stream, p);
       PA_CHECK_LAUNCH("attention kernel (bounded scores)");
+    }
+  }
+  if constexpr (D == 128 && SPARSE) {
+    if (p.pair) {
+      const void* fp = (const void*)attn_fwd_d128_pipe_kernel<T, true, 8, false, true>;
+      if (dev < 0 || !attr_done[dev][5]) {
+        hipError_t e = hipFuncSetAttribute(fp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        if (dev >= 0) attr_done[dev][5] = true;
+      }
+      hipLaunchKernelGGL((attn_fwd_d128_pipe_kernel<T, true, 8, false, true>), dim3((unsigned)nblocks), dim3(512), smem, stream, p);
+      PA_CHECK_LAUNCH("attention kernel (paired query blocks)");
+      return PA_OK;
     }
   }
   if constexpr (D == 128) {
@@ -2728,8 +2859,9 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
 //   PARAATTN_BOUND=0|1       "bound"         never / always compute the score bound (-1 = by size)
 //   PARAATTN_STREAM=0|1      "stream"        never / wherever possible the resident-workgroup kernel (-1 = by shape)
 //   PARAATTN_STREAM_EVEN=0|1 "stream_even"   its tail cut into shares that begin at the same keys / into equal ranges (-1 = by size)
+//   PARAATTN_SPARSE_PAIR=1   "sparse_pair"   block-sparse with 128-row query blocks: two adjacent blocks per 256-row workgroup
 struct Tuning {
-  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even;
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair;
 };
 static Tuning& tuning() {
   static Tuning t;
@@ -2748,6 +2880,7 @@ static Tuning& tuning() {
     t.stream = st == 0 || st == 1 ? st : -1;
     const int se = num("PARAATTN_STREAM_EVEN", -1);
     t.stream_even = se == 0 || se == 1 ? se : -1;
+    t.sparse_pair = num("PARAATTN_SPARSE_PAIR", 0) == 1;
     return true;
   }();
   (void)init;
@@ -2766,6 +2899,7 @@ extern "C" int pa_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bound")) t.bound = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "stream")) t.stream = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "stream_even")) t.stream_even = value == 0 || value == 1 ? value : -1;
+  else if (!strcmp(name, "sparse_pair")) t.sparse_pair = value == 1;
   else PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: unknown knob '%s'", name);
   return PA_OK;
 }
@@ -3281,11 +3415,21 @@ extern "C" int pa_attn_fwd_lse_noalloc(const void* q, const void* k, const void*
                         out_strides, scale, kv_len, is_causal, ws, ws ? (size_t)PA_NOALLOC_SCRATCH_BYTES : 0, stream);
 }
 
+// The lists of paired query blocks (build_pair_runs_kernel): half the segments, up to nK + 2 ranges each.
+static size_t pair_runs_bytes(int Hm, int nQ, int nK) {
+  const size_t nseg = (size_t)nQ / 2 + 2;
+  const size_t cap = (size_t)nK + 3;
+  return sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2);
+}
+
+// Room for either form of the lists (per query block: up to nK / 2 + 2 ranges each; per pair of query blocks).
 extern "C" size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK) {
   if (Hm <= 0 || nQ <= 0 || nK <= 0) return 0;
   const size_t nseg = (size_t)nQ + 2;
   const size_t cap = (size_t)nK / 2 + 3;
-  return sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2);
+  const size_t single = sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2);
+  const size_t pairs = pair_runs_bytes(Hm, nQ, nK);
+  return single > pairs ? single : pairs;
 }
 
 extern "C" int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int nQ, int nK, int Skv,
@@ -3311,13 +3455,24 @@ static int blocksparse_launch(const void* q, const void* k, const void* v, void*
                               int B, int H, int Sq, int Skv, int D, const int64_t q_strides[3],
                               const int64_t k_strides[3], const int64_t v_strides[3],
                               const int64_t out_strides[3], float scale, int Hm, int nQ, int nK, int q_lo,
-                              int q_block, const int32_t* runs, void* stream) {
+                              int q_block, const int32_t* runs, void* stream, bool pair = false) {
   AttnParams p;
   fill_params(p, q, k, v, out, lse, B, H, Sq, Skv, q_strides, k_strides, v_strides, out_strides, scale);
   p.runs = runs;
   p.Hm = Hm; p.nQ = nQ; p.cap = nK / 2 + 3;
   p.q_lo = q_lo; p.q_block = q_block;
   choose_kernel(p, D, (q_block % 256 == 0 && q_lo % 256 == 0) ? 256 : 128, false, 0, nullptr);
+  if (pair) {  // `runs` holds the lists of pairs: 256-row workgroups over nQ / 2 double blocks
+    if (!p.pipe || D != 128 || q_block != 128 || nQ % 2 != 0 || q_lo % 256 != 0)
+      PA_FAIL(PA_ERR_UNSUPPORTED, "paired query blocks need the pipelined head_dim-128 kernel, 128-row blocks in even number from a multiple of 256");
+    p.pair = 1;
+    p.bm = 256;
+    p.nQ = nQ / 2;
+    p.q_block = 256;
+    p.cap = nK + 3;
+    nQ = p.nQ;
+    q_block = 256;
+  }
   p.tiles_left = (q_lo + p.bm - 1) / p.bm;
   p.tiles_per_block = (q_block + p.bm - 1) / p.bm;
   const int q_hi = q_lo + nQ * q_block;
@@ -3350,6 +3505,19 @@ extern "C" int pa_attn_fwd_blocksparse(const void* q, const void* k, const void*
   int rc = blocksparse_check(q, k, v, out, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
                              scale, Hm, nQ, nK, q_lo, q_block);
   if (rc) return rc;
+  // two 128-row query blocks per workgroup (tuning knob, off by default): their own lists in the same workspace
+  const uint64_t kv_span = Skv > 0 ? (uint64_t)(Skv - 1) * 2 : 0;
+  if (tuning().sparse_pair && !tuning().no_pipe && D == 128 && q_block == 128 && nQ % 2 == 0 && q_lo % 256 == 0 &&
+      kv_lo % 4 == 0 && kv_block % 4 == 0 && Skv % 4 == 0 && Skv > 0 && block_mask && runs_ws && kv_block > 0 &&
+      kv_lo >= 0 && (int64_t)kv_lo + (int64_t)nK * kv_block <= Skv &&
+      kv_span * (uint64_t)k_strides[2] + 256 < PIPE_OOB && kv_span * (uint64_t)v_strides[2] + 256 < PIPE_OOB &&
+      runs_ws_bytes >= pair_runs_bytes(Hm, nQ, nK)) {
+    hipLaunchKernelGGL(build_pair_runs_kernel, dim3(Hm * (nQ / 2 + 2)), dim3(64), 0, (hipStream_t)stream,
+                       block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, nK + 3, runs_ws);
+    PA_CHECK_LAUNCH("build_pair_runs_kernel");
+    return blocksparse_launch(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,
+                              out_strides, scale, Hm, nQ, nK, q_lo, q_block, runs_ws, stream, true);
+  }
   rc = pa_blocksparse_build_runs(block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, runs_ws, runs_ws_bytes, stream);
   if (rc) return rc;
   return blocksparse_launch(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides,

@@ -149,6 +149,45 @@ def test_prebuilt_runs_entry(cuda):
         assert torch.equal(o3, want3) and len(cache) == 1 and next(iter(cache.values())) is not held
 
 
+def test_paired_query_blocks(cuda, tuning):
+    """Two adjacent 128-row query blocks in one 256-row workgroup over the union of their key ranges (tuning knob
+    "sparse_pair"): the same results as one workgroup per block to the kernels' tolerance, and as float64 dense
+    attention over the kept tiles; with margins, per-head masks, rows of a pair that keep nothing, key blocks
+    smaller than a tile."""
+    rng = np.random.default_rng(5)
+    op = torch.ops.para_attn.attention_forward_block_sparse
+    for case, (H, nQ, nK, kb, q_lo, q_tail, kv_lo, kv_tail, dens, per_head) in enumerate([
+        (2, 4, 6, 128, 0, 0, 0, 0, 0.5, True),
+        (3, 6, 9, 64, 256, 37, 24, 12, 0.4, True),
+        (1, 2, 5, 100, 0, 130, 8, 0, 0.3, False),
+        (2, 8, 16, 32, 0, 0, 0, 64, 0.25, True),
+        (2, 4, 4, 128, 0, 0, 0, 0, 1.0, False),
+    ]):
+        Sq, Skv = q_lo + nQ * 128 + q_tail, kv_lo + nK * kb + kv_tail
+        bm = torch.from_numpy(rng.random((H if per_head else 1, nQ, nK)) < dens)
+        if case == 1:
+            bm[:, 3] = False  # the upper block of a pair keeps nothing (margins aside)
+        bm2 = bm if per_head else bm[0]
+        q, k, v = inputs.qkv(1, H, Sq, Skv, 128, seed=900 + case)
+        q_range, kv_range = (q_lo, q_lo + nQ * 128), (kv_lo, kv_lo + nK * kb)
+        keep = osparse.expand_block_mask(bm2.numpy(), Sq, Skv, q_range, kv_range)
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, keep)
+        args = (q.to(cuda), k.to(cuda), v.to(cuda), bm2.to(cuda), *q_range, *kv_range)
+        tuning("sparse_pair", 0)
+        out0, lse0 = op(*args)
+        tuning("sparse_pair", 1)
+        out1, lse1 = op(*args)
+        tuning("sparse_pair", 0)
+        what = f"case {case}"
+        got_lse, got_out = lse1.cpu().numpy(), out1.float().cpu().numpy()
+        dead = np.isneginf(ref_lse)
+        assert (np.isneginf(got_lse) == dead).all(), what
+        np.testing.assert_allclose(np.where(dead, 0, got_lse), np.where(dead, 0, ref_lse), atol=1e-3, err_msg=what)
+        np.testing.assert_allclose(got_out, np.where(dead[..., None], 0, ref_out), atol=2e-2, rtol=2e-2, err_msg=what)
+        assert (np.where(dead, 0, got_lse - lse0.cpu().numpy()) == 0).all() or np.abs(np.where(dead, 0, got_lse - lse0.cpu().numpy())).max() < 1e-4, what
+        assert (out1.float() - out0.float()).abs().max().item() <= 2e-2, what
+
+
 def test_row_without_kept_block(cuda):
     # the reference asserts out on such a row (torch _SDPAMerger.results() with nothing merged);
     # the kernel defines it: out = 0, lse = -inf
