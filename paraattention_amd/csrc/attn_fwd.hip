@@ -1958,13 +1958,14 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   const uint32_t v_off0 = dma_row * vs_bytes + 16 * (dma_pc ^ (4 * (dma_row & 3)));
   const uint32_t lds_k = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sK + wave * 1024);
   const uint32_t lds_v = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sV + wave * 1024);
-  auto dma_k1 = [&](int buf, uint32_t n0, int i) __attribute__((always_inline)) {
-    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * ks_bytes);
+  // `there`: the tile is known to exist (no test for OOB)
+  auto dma_k1 = [&](int buf, uint32_t n0, int i, bool there = false) __attribute__((always_inline)) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(!there && n0 == OOB ? OOB : (n0 + RS * i) * ks_bytes);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_k + buf * TILE_BYTES + i * (RS * 256)), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
   };
-  auto dma_v1 = [&](int buf, uint32_t n0, int i) __attribute__((always_inline)) {
-    const uint32_t soff = __builtin_amdgcn_readfirstlane(n0 == OOB ? OOB : (n0 + RS * i) * vs_bytes);
+  auto dma_v1 = [&](int buf, uint32_t n0, int i, bool there = false) __attribute__((always_inline)) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane(!there && n0 == OOB ? OOB : (n0 + RS * i) * vs_bytes);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_v + buf * TILE_BYTES + i * (RS * 256)), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
   };
@@ -2143,9 +2144,12 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   // the scores of the second tile already belong to another piece: its Q replaces the first piece's
   if (nxt.piece >= 0 && nxt.piece != cur.piece) load_q(nxt.piece);
 
-  // One iteration; PAR = buffer of tile j (K(j+1) sits in the other K buffer).
-  auto tile_step = [&](auto PAR) __attribute__((always_inline)) {
+  // One iteration; PAR = buffer of tile j (K(j+1) sits in the other K buffer).  INSIDE: tiles j .. j+3 are
+  // whole tiles of one item and one segment, none of them the item's last: nothing but the tile itself happens,
+  // and the window moves on by 64 keys.
+  auto tile_step = [&](auto PAR, auto INSIDE) __attribute__((always_inline)) {
     constexpr int par = decltype(PAR)::value;
+    constexpr bool inside = decltype(INSIDE)::value;
     const char* tV = sV + par * TILE_BYTES;
     const char* tKn = sK + (par ^ 1) * TILE_BYTES;
     floatx16 c0 = sn0, c1 = sn1;  // S(j)
@@ -2200,8 +2204,8 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
     for (int g = 0; g < 8; ++g) {
       if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
       else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
-      if (g < IPW) dma_k1(par, nx2.n0, g);
-      else if (g < 2 * IPW) dma_v1(par ^ 1, nxt.n0, g - IPW);
+      if (g < IPW) dma_k1(par, nx2.n0, g, inside);
+      else if (g < 2 * IPW) dma_v1(par ^ 1, nxt.n0, g - IPW, inside);
       f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
       expo_slot(g);
       __builtin_amdgcn_sched_barrier(0);
@@ -2214,12 +2218,12 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
       if (g < 4) expo_slot(8 + g);
       __builtin_amdgcn_sched_barrier(0);
     }
-    {
+    if constexpr (!inside) {
       const int nv1 = valid_keys(nxt.n0);
       if (nv1 < BN) mask_tail(sn0, sn1, nv1);  // ragged or absent tile j+1
+      // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
+      if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
     }
-    // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
-    if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage B: O^T += V(j)^T P(j)^T, the rest of the softmax, the row maximum of S(j+1) ----------
@@ -2259,24 +2263,51 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
     l_run += lsum;
     if constexpr (!BOUNDED) mx = across(fmaxf(mxa, mxb));
 
-    if (cur.flags & LAST) finish_item(cur);
+    if constexpr (inside) {
+      cur.n0 = nxt.n0;
+      nxt.n0 = nx2.n0;
+      nx2.n0 += BN;
+    } else {
+      if (cur.flags & LAST) finish_item(cur);
 
-    // slide the tile window and point the descriptors at what the next iteration copies (this iteration's
-    // copies are all issued); done here, under the last MFMAs, and not behind the next barrier, where every
-    // wavefront of the workgroup would wait for it
-    cur = nxt;
-    nxt = nx2;
-    pull(nx2);
-    aim_k(nx2);
-    aim_v(nxt);
+      // slide the tile window and point the descriptors at what the next iteration copies (this iteration's
+      // copies are all issued); done here, under the last MFMAs, and not behind the next barrier, where every
+      // wavefront of the workgroup would wait for it
+      cur = nxt;
+      nxt = nx2;
+      pull(nx2);
+      aim_k(nx2);
+      aim_v(nxt);
+    }
+  };
+  // How many of the coming iterations are INSIDE ones: the window lies in one piece and segment (so tile j is not
+  // an item's last, tile j+1 is whole, no Q or descriptor changes), and the tiles the generator hands out next
+  // stay in that item and segment without being the last of either (their descriptors differ from tile j+2's in
+  // the first key only).
+  auto inside_run = [&]() __attribute__((always_inline)) {
+    if (nx2.piece < 0 || cur.piece != nx2.piece || cur.seg != nx2.seg || g_jj == 0) return 0;
+    const int a = g_jend - 1 - g_j, b = sp.tps - 1 - g_jj;
+    const int n = a < b ? a : b;
+    return n > 0 ? n : 0;
   };
 
   aim_k(nx2);
   aim_v(nxt);
+  constexpr std::integral_constant<int, 0> even{};
+  constexpr std::integral_constant<int, 1> odd{};
   while (cur.piece >= 0) {
-    tile_step(std::integral_constant<int, 0>{});
+    int pairs = inside_run() >> 1;
+    if (pairs > 0) {
+      g_j += 2 * pairs;  // the generator hands these tiles out in one go
+      g_jj += 2 * pairs;
+      do {
+        tile_step(even, std::true_type{});
+        tile_step(odd, std::true_type{});
+      } while (--pairs > 0);
+    }
+    tile_step(even, std::false_type{});
     if (cur.piece < 0) break;
-    tile_step(std::integral_constant<int, 1>{});
+    tile_step(odd, std::false_type{});
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the wavefront ends
 }
