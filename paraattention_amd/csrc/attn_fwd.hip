@@ -1800,7 +1800,10 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   const int l32 = lane & 31;
   const int hh = lane >> 5;
   const StreamPlan& sp = p.st;
-  const int wg = blockIdx.x;
+  // Workgroups are dealt to the 8 XCDs in turn; with G a multiple of 8 each XCD takes a contiguous eighth of the
+  // workgroup numbers, so the pieces its 32 workgroups sweep at one time are neighbours (one or two heads, whose
+  // K/V tiles then meet in that XCD's L2), and so are its ranges of the tail.
+  const int wg = (sp.G & 7) == 0 ? (int)(blockIdx.x & 7) * (sp.G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
   constexpr uint32_t OOB = PIPE_OOB;
   // What happens once per piece (a new Q, a new K/V descriptor, a finished piece's output) needs many of the
   // kernel's arguments and little else.  Read through `p` the compiler would load them all once, ahead of the
