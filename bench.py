@@ -34,7 +34,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Traffic at the L2's memory side per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two
 # rocprofv3 --pmc runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy).  These counters cannot be
 # read from inside this process; the figures are those of the summary named in TRAFFIC_SOURCE, not of this run.
-TRAFFIC = {"attn": 4.136e9, "merge": 4.632e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 1.931e10}
+TRAFFIC = {"attn": 4.137e9, "merge": 4.775e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 1.914e10,
+           "flux": 6.55e8, "ring_sweep": 1.427e10, "ring_sweep_per_block": 1.847e10, "wan_self": 6.066e9, "wan_cross": 7.79e8}
 TRAFFIC_SOURCE = "profiles/kernels_bench_workloads.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the same command)"
 
 
@@ -135,7 +136,7 @@ def bench_attn(dev, steps, warmup):
     return (q, k, v), 4.0 * B * H * S * S * D, t, checked
 
 
-def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=(0,)):
+def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=(0,), traffic=None):
     import torch
 
     from oracle import inputs
@@ -154,19 +155,20 @@ def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=
     flops = 4.0 * B * H * Sq * Skv * D
     nbytes = 2.0 * B * H * D * (2 * Sq + 2 * Skv) + 4.0 * B * H * Sq
     gbs = nbytes / (t["median"] * 1e-3) / 1e9
+    more = {"traffic": TRAFFIC[traffic], "traffic_source": TRAFFIC_SOURCE} if traffic else {}
     return _mfma(f"{name}: attention_forward_with_lse q [{B},{H},{Sq},{D}] k,v [{B},{H},{Skv},{D}] bf16", flops, t,
-                 bytes=nbytes, gbs=round(gbs, 1), frac_hbm=round(gbs / PEAK_HBM_GBS, 4), checked=checked)
+                 bytes=nbytes, gbs=round(gbs, 1), frac_hbm=round(gbs / PEAK_HBM_GBS, 4), checked=checked, **more)
 
 
 def bench_flux(dev, steps=20, warmup=5):
-    return _dense_case(dev, "FLUX joint attention", 1, 24, 4608, 4608, 128, steps, warmup, seed=0)
+    return _dense_case(dev, "FLUX joint attention", 1, 24, 4608, 4608, 128, steps, warmup, seed=0, traffic="flux")
 
 
 def bench_wan(dev, steps=10, warmup=3):
     """Both attention legs of a Wan 2.1 block.  Cross-attention to 512 keys sits near the ridge: both bounds."""
     return {
-        "wan_self_attention": _dense_case(dev, "Wan 2.1 self-attention", 1, 40, 32760, 32760, 128, steps, warmup, seed=4, check_heads=(0, 17)),
-        "wan_cross_attention": _dense_case(dev, "Wan 2.1 cross-attention to 512 text keys", 1, 40, 32760, 512, 128, 2 * steps, warmup, seed=2, check_heads=(0, 17)),
+        "wan_self_attention": _dense_case(dev, "Wan 2.1 self-attention", 1, 40, 32760, 32760, 128, steps, warmup, seed=4, check_heads=(0, 17), traffic="wan_self"),
+        "wan_cross_attention": _dense_case(dev, "Wan 2.1 cross-attention to 512 text keys", 1, 40, 32760, 512, 128, 2 * steps, warmup, seed=2, check_heads=(0, 17), traffic="wan_cross"),
     }
 
 
@@ -202,7 +204,7 @@ def bench_ring(dev, steps=5, warmup=2):
         t = _time_calls(call, steps, warmup)
         checked = _check_rows(last["out"][:, heads], last["lse"][:, heads], q[:, heads], k_all, v_all, [0, 1], _sample_rows(S), key)
         out[key] = _mfma(f"ring sweep: Q block [1,24,14882,128] bf16 against 8 KV blocks of 14882 keys, {how}", flops, t,
-                         launches_per_sweep=launches, checked=checked)
+                         launches_per_sweep=launches, checked=checked, traffic=TRAFFIC[key], traffic_source=TRAFFIC_SOURCE)
     return out
 
 
@@ -430,7 +432,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "pa::attn_fwd_d128_pipe_kernel<pa::BF16, false, 8, true>",
+            "kernel": "pa::attn_fwd_d128_pipe_kernel<pa::BF16, false, 8, true, false>",
             "achieved": round(kern_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
