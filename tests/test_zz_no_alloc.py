@@ -72,6 +72,7 @@ def test_noalloc_matches_workspace_entry_on_two_calls(cuda, tuning):
 def test_noalloc_refuses_what_the_buffer_cannot_hold(cuda, tuning):
     lib = _lib.load()
     tuning("bm", 256)
+    tuning("stream", 0)  # the key-split plan (the resident-workgroup plan keeps these 150 pieces whole and needs nothing)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     # one head, a round and 150 query tiles more, long keys: the plan splits the 150 tiles' keys several ways
     B, H, D, Sq, Skv = 1, 1, 128, (cus + 150) * 256, 16384
