@@ -2,8 +2,8 @@
 (B=1, 3 of 24 heads, S=119056, D=128, bf16, q/k RMS-normalised), one MI355X.
 
 Prints ONE JSON line.  ``value`` is attention TFLOP/s (4*B*H*Sq*Skv*D flop per call) with inputs
-resident in HBM (a call = everything the op launches: the score bound's two small kernels, the
-attention kernel and the merge of its key-split tail); ``roofline`` prices the call against the bf16
+resident in HBM (a call = everything the op launches: the score bound's two small kernels, both
+variants of the attention kernel, one of which returns at once, and the merge of the partial results); ``roofline`` prices the call against the bf16
 dense MFMA peak; ``cpu_baseline`` is torch's CPU SDPA (the library routine the reference's SDPA path
 is checked against) on a bounded sample of the same workload; ``extras`` holds the other
 configurations of the baseline (FLUX joint attention, the ring sweep, the Wan self- and
@@ -11,7 +11,11 @@ cross-attention legs, block-sparse attention) against the MFMA peak and the band
 (ring merge step, FBCache reduction, TaylorSeer) against the HBM peak.
 
 Every timed loop takes per-call HIP events on the launch stream and reports mean, median and
-minimum; the bandwidth-bound kernels rotate over several buffer sets so that the 256 MB
+minimum.  What is reported is the steady state of a loop that keeps the GPU busy, which is what a diffusion
+model's step is: after an idle gap the chip needs some tenths of a second of work to settle (measured: the
+headline call takes 17.61 ms after 3 warm-up calls, 17.50 after 10, 17.40 after 30; FLUX joint attention 0.298 ms
+after 5, 0.258 after 50, 0.255 after 200; the bandwidth-bound kernels move the other way, 2-3 % faster right after
+the gap), so the defaults warm every loop up for that long (30 calls of the headline, 60-100 of the short kernels); the bandwidth-bound kernels rotate over several buffer sets so that the 256 MB
 memory-side cache cannot hold a working set from one call to the next; a sample of rows of the last
 timed output of every attention shape is compared with torch's CPU SDPA (``checked``).
 
@@ -160,19 +164,19 @@ def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=
                  bytes=nbytes, gbs=round(gbs, 1), frac_hbm=round(gbs / PEAK_HBM_GBS, 4), checked=checked, **more)
 
 
-def bench_flux(dev, steps=20, warmup=5):
+def bench_flux(dev, steps=50, warmup=100):
     return _dense_case(dev, "FLUX joint attention", 1, 24, 4608, 4608, 128, steps, warmup, seed=0, traffic="flux")
 
 
-def bench_wan(dev, steps=10, warmup=3):
+def bench_wan(dev, steps=10, warmup=10):
     """Both attention legs of a Wan 2.1 block.  Cross-attention to 512 keys sits near the ridge: both bounds."""
     return {
         "wan_self_attention": _dense_case(dev, "Wan 2.1 self-attention", 1, 40, 32760, 32760, 128, steps, warmup, seed=4, check_heads=(0, 17), traffic="wan_self"),
-        "wan_cross_attention": _dense_case(dev, "Wan 2.1 cross-attention to 512 text keys", 1, 40, 32760, 512, 128, 2 * steps, warmup, seed=2, check_heads=(0, 17), traffic="wan_cross"),
+        "wan_cross_attention": _dense_case(dev, "Wan 2.1 cross-attention to 512 text keys", 1, 40, 32760, 512, 128, 4 * steps, 10 * warmup, seed=2, check_heads=(0, 17), traffic="wan_cross"),
     }
 
 
-def bench_ring(dev, steps=5, warmup=2):
+def bench_ring(dev, steps=6, warmup=3):
     """One rank's ring pass: a Q block of 14882 tokens x 24 heads against 8 KV blocks of 14882 keys; checked against
     one SDPA over all 119056 keys.  Two ways: all blocks in one launch (the softmax state carried across the blocks
     in registers: what a sweep over resident blocks is), and one launch per block with the fp32 running pair folded
@@ -230,7 +234,7 @@ def bench_shapes(dev, steps=10, warmup=3):
     return rows
 
 
-def bench_sparse(dev, steps=10, warmup=5):
+def bench_sparse(dev, steps=10, warmup=10):
     import torch
 
     from oracle import inputs
@@ -274,7 +278,7 @@ def bench_sparse(dev, steps=10, warmup=5):
 SETS = 3
 
 
-def bench_merge(dev, steps=21, warmup=3):
+def bench_merge(dev, steps=30, warmup=60):
     import torch
 
     # ring merge step at the ring-sweep shape: fp32 accumulator updated in place by a bf16 partial
@@ -290,7 +294,7 @@ def bench_merge(dev, steps=21, warmup=3):
     return _hbm("merge", "ring merge step: fp32 acc [1,24,14882,128] updated in place by a bf16 partial + fp32 LSE", nbytes, t, SETS)
 
 
-def bench_fbcache(dev, steps=21, warmup=3):
+def bench_fbcache(dev, steps=30, warmup=60):
     from oracle import fbcache as ofb
     from oracle import inputs
 
@@ -314,7 +318,7 @@ def bench_fbcache(dev, steps=21, warmup=3):
     return r
 
 
-def bench_taylorseer(dev, steps=12, warmup=3):
+def bench_taylorseer(dev, steps=30, warmup=60):
     import torch
 
     # cache-hit step with TaylorSeer on: value of 3 stored orders + hidden states, one pass
@@ -383,8 +387,8 @@ def cpu_baseline(q, k, v):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=None, help="timed calls (default: 20 for the headline, each extra's own otherwise)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed calls before them (default: 30 for the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     singles = {"merge": bench_merge, "fbcache": bench_fbcache, "taylorseer": bench_taylorseer, "sparse": bench_sparse,
@@ -405,10 +409,13 @@ def main():
     dev = torch.device("cuda:0")
 
     if args.only in singles:
-        print(json.dumps({args.only: singles[args.only](dev, args.steps, args.warmup)}))
+        given = {k: v for k, v in (("steps", args.steps), ("warmup", args.warmup)) if v is not None}
+        print(json.dumps({args.only: singles[args.only](dev, **given)}))
         return
 
-    (q, k, v), flops, t, checked = bench_attn(dev, args.steps, args.warmup)
+    steps = 20 if args.steps is None else args.steps
+    warmup = 30 if args.warmup is None else args.warmup
+    (q, k, v), flops, t, checked = bench_attn(dev, steps, warmup)
     tflops = flops / (t["wall"] * 1e-3) / 1e12
     kern_tflops = flops / (t["mean"] * 1e-3) / 1e12
     result = {
@@ -416,8 +423,8 @@ def main():
         "value": round(tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(t["wall"], 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -432,7 +439,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "pa::attn_fwd_d128_pipe_kernel<pa::BF16, false, 8, true, false>",
+            "kernel": "pa::attn_fwd_d128_stream_kernel<pa::BF16, true>",
             "achieved": round(kern_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",

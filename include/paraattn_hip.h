@@ -165,7 +165,7 @@ PA_API size_t pa_attn_fwd_masked_workspace_bytes(int B, int H, int Sq, int Skv, 
  * between calls and nothing has to be cleared; but all calls on one GPU share
  * it, so calls that overlap on one GPU (two streams, two threads) race.
  */
-#define PA_NOALLOC_SCRATCH_BYTES (64u << 20)
+#define PA_NOALLOC_SCRATCH_BYTES (80u << 20)
 PA_API int pa_attn_fwd_lse_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
                             int dtype, int B, int H, int Sq, int Skv, int D,
                             const int64_t q_strides[3], const int64_t k_strides[3],

@@ -22,7 +22,7 @@ PA_DTYPE_BF16 = 0
 PA_DTYPE_F16 = 1
 PA_DTYPE_F32 = 2
 
-PA_NOALLOC_SCRATCH_BYTES = 64 << 20
+PA_NOALLOC_SCRATCH_BYTES = 80 << 20
 
 PA_MASK_BOOL = 1
 PA_MASK_F32 = 2

@@ -2210,7 +2210,6 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
       if (g < IPW) dma_k1(par, nx2.n0, g, inside);
       else if (g < 2 * IPW) dma_v1(par ^ 1, nxt.n0, g - IPW, inside);
       f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
-      expo_slot(g);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -2218,7 +2217,6 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
       if (g & 1) sn1 = T::mfma32(f[g], qf[4 + (g >> 1)], sn1);
       else sn0 = T::mfma32(f[g], qf[4 + (g >> 1)], sn0);
       f[g] = read_vt(tV, 0, g >> 2, g & 3);
-      if (g < 4) expo_slot(8 + g);
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (!inside) {
@@ -2227,6 +2225,12 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
       // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
       if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
     }
+    __builtin_amdgcn_sched_barrier(0);
+    // The softmax of S(j) begins here, not under the MFMAs of stage A: VALU work between the MFMAs of the first
+    // GEMM costs more than it hides (measured in attn_fwd_d128_pipe_kernel, where the compiler makes this same
+    // arrangement by itself): 22 of the 32 exponentials in front of the first PV MFMA, the other 10 under them.
+#pragma unroll
+    for (int n = 0; n < 6; ++n) expo_slot(n);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- stage B: O^T += V(j)^T P(j)^T, the rest of the softmax, the row maximum of S(j+1) ----------
@@ -2240,7 +2244,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
         f[g] = read_vt(tV, 1, cc, db);
-        if (g < 6) expo_slot(12 + g);
+        expo_slot(6 + g);
         if constexpr (!BOUNDED) {
           if (g < 4) {
           } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
@@ -2257,6 +2261,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
       for (int db = 0; db < DB; ++db) {
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
+        if (g < 4) expo_slot(14 + g);
         if constexpr (!BOUNDED) {
           if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
         }
@@ -3038,7 +3043,7 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   *ws_need = 0;
   const bool multi = segs != nullptr;
   const int want = tuning().stream;
-  if (want == 0 || (multi && want < 0)) return false;  // key segments: attn_fwd_d128_pipe_kernel walks them too, faster on long sweeps
+  if (want == 0 || (want < 0 && tuning().forced_bm != 0)) return false;  // switched off, or a workgroup size of the other kernels asked for
   if (D != 128 || p.causal || p.kv_len != nullptr || tuning().no_pipe) return false;
   const int cus = device_cus();
   if (cus <= 0) return false;
@@ -3052,18 +3057,10 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   const int64_t P64 = (int64_t)p.B * p.H * nqt;
   if (L64 > 0x3fffffff || P64 > 0x3fffffff) return false;
   const int L = (int)L64, P = (int)P64;
-  // Where it pays (measured).  A workgroup per piece spends about 11 key tiles' time on what is not the key
-  // sweep, and a partly filled last round idles the chip; resident workgroups hide the first and cut the second
-  // finely.  But their loop carries more scalar bookkeeping per key tile (15 % more clocks per tile, which the
-  // power-limited chip answers with 8 % more clock: 5-7 % slower per tile), so they win where pieces are short
-  // (up to 16 key tiles: cross-attention to a text prompt) or the launch has fewer than two rounds of pieces and
-  // the last one is partly filled (image models: FLUX has 1.7), and lose on long launches of many rounds.
-  if (!multi && want < 0) {
-    const int rounds = P / cus, left = P % cus;
-    const bool short_pieces = L <= 16 && P >= 2 * cus;
-    const bool ragged_rounds = rounds <= 1 && left > 0 && (int64_t)P * L >= 16 * (int64_t)cus;
-    if (!short_pieces && !ragged_rounds) return false;
-  }
+  // Taken wherever it applies (measured against attn_fwd_d128_pipe_kernel + key-split tail on one box: 119056 keys
+  // +0.6 %, Wan self-attention +0.9 %, a ring sweep's block +3.5 %, the sweep in one launch +1.3 %, 16k / 8k / 6k /
+  // 3k tokens +1.5 / +2.4 / +7 / +7 %, FLUX +10..17 %, cross-attention to 512 keys +6 %): the hot loop is the same,
+  // and resident workgroups hide what a workgroup per piece pays per piece and cut a ragged last round finely.
   StreamPlan& st = p.st;
   st.G = cus;
   st.R = P / st.G;
@@ -3080,10 +3077,10 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   st.Gt = 0;
   if (p_tail > 0) {
     const int64_t t_tail = (int64_t)p_tail * L;
-    // K and V of one head: where the L2s hold that (4 MB each), workgroups need not sweep the keys in step
-    const double head_bytes = (double)L * BN * ((double)p.ks_s + (double)p.vs_s) * 2.0;
+    // equal ranges by default: shares of whole pieces that begin at the same keys keep the tail's workgroups in step
+    // on the keys, but leave workgroups idle; measured slower or equal at every shape from 3000 to 119056 keys
     const int ev = tuning().stream_even;
-    const bool even = ev >= 0 ? ev == 1 : head_bytes <= 6.0e6;
+    const bool even = ev != 0;
     int gt;
     if (even) {
       const int64_t by_size = t_tail / 8;  // at least 8 key tiles per workgroup
@@ -3096,10 +3093,17 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
       gt = p_tail * sh;
     }
     if (tuning().no_split) gt = p_tail;
-    size_t need = gt != p_tail ? (size_t)2 * gt * 256 * (128 + 1) * sizeof(float) : 0;
-    if (need > ws_avail && !sizing) {  // whole pieces only
-      gt = p_tail;
-      need = 0;
+    const size_t per_range = (size_t)2 * 256 * (128 + 1) * sizeof(float);  // two partial results per workgroup
+    size_t need = gt != p_tail ? gt * per_range : 0;
+    if (need > ws_avail && !sizing) {  // as many ranges as the workspace holds, if that still beats whole pieces
+      const int64_t fit = (int64_t)(ws_avail / per_range);
+      if (even && fit > p_tail) {
+        gt = (int)fit;
+        need = gt * per_range;
+      } else {
+        gt = p_tail;
+        need = 0;
+      }
     }
     st.Gt = gt;
     *ws_need = need;
@@ -3308,16 +3312,33 @@ extern "C" size_t pa_attn_fwd_sweep_workspace_bytes(int B, int H, int Sq, int n_
   return need;
 }
 
+// Workspace of a dense call: partial results of the plan plus the score bound's words.  which = 0: the plan of a
+// call without per-batch key counts and is_causal (resident workgroups where they apply); 1: the plan of a call
+// with either; 2: the larger.
+static size_t dense_ws_need(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3], const int64_t v_strides[3], int which) {
+  const int64_t zero[3] = {0, 0, 0};
+  size_t best = 0;
+  for (int plan = 0; plan < 2; ++plan) {
+    if (which != 2 && which != plan) continue;
+    AttnParams p;
+    fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
+    size_t need = 0;
+    if (plan == 1 || !plan_stream(p, D, nullptr, 0, true, &need)) {
+      need = 0;
+      choose_kernel(p, D, 256, true, 0, &need);
+    }
+    if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && (D == 64 || p.bm == 256)) need += BOUND_WS_BYTES;
+    if (need > best) best = need;
+  }
+  return best;
+}
+
 extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
                                               const int64_t k_strides[3], const int64_t v_strides[3]) {
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || (D != 128 && D != 64) || !k_strides || !v_strides) return 0;
-  AttnParams p;
-  const int64_t zero[3] = {0, 0, 0};
-  fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
-  size_t need = 0;
-  if (!plan_stream(p, D, nullptr, 0, true, &need)) choose_kernel(p, D, 256, true, 0, &need);
-  if (bound_wanted(B, H, Sq, Skv, D) && p.pipe && (D == 64 || p.bm == 256)) need += BOUND_WS_BYTES;
-  return need;
+  // the larger of what the two plans ask for: which of them a call gets depends on arguments this function does not
+  // see (per-batch key counts and is_causal go to attn_fwd_d128_pipe_kernel)
+  return dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, 2);
 }
 
 // The generic kernel with an attention mask (any head_dim it is built for, any strides).
@@ -3436,7 +3457,8 @@ extern "C" int pa_attn_fwd_lse_noalloc(const void* q, const void* k, const void*
                                        const int64_t v_strides[3], const int64_t out_strides[3],
                                        float scale, const int32_t* kv_len, int is_causal, void* stream) {
   // what the same problem would ask of a caller's workspace (0 for sizes that use none)
-  const size_t need = (k_strides && v_strides) ? pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, k_strides, v_strides) : 0;
+  const bool shaped = B > 0 && H > 0 && Sq > 0 && Skv > 0 && (D == 128 || D == 64) && k_strides && v_strides;
+  const size_t need = shaped ? dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, kv_len != nullptr || is_causal ? 1 : 0) : 0;
   if (need > (size_t)PA_NOALLOC_SCRATCH_BYTES)
     PA_FAIL(PA_ERR_WORKSPACE, "this problem's launch plan needs %zu bytes of scratch, the static buffer holds %zu: "
             "call pa_attn_fwd_lse_ws with a workspace of your own", need, (size_t)PA_NOALLOC_SCRATCH_BYTES);

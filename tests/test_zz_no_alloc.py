@@ -69,6 +69,26 @@ def test_noalloc_matches_workspace_entry_on_two_calls(cuda, tuning):
     assert first_need > 16384, "the first shape is meant to take the key-split path (partials in the scratch)"
 
 
+def test_noalloc_with_resident_workgroups(cuda, tuning):
+    """The default plan of a dense call (resident workgroups, the ragged last round cut into ranges whose partial
+    results lie in the scratch): bit for bit the workspace entry's result, on two calls in a row."""
+    lib = _lib.load()
+    tuning("bound", 1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    B, D = 1, 128
+    for H, Sq, Skv in ((4, (cus // 4 + 25) * 256 - 50, 64 * 30 + 11), (3, 9 * 256 + 3, 64 * 9)):
+        q, k, v = (t.to(cuda) for t in inputs.qkv(B, H, Sq, Skv, D, seed=Sq))
+        want_out, want_lse, need = _call_ws(lib, q, k, v)
+        assert need > 16384, "meant to cut pieces (partial results in the workspace)"
+        rc, out, lse = _call_noalloc(lib, q, k, v)
+        assert rc == 0, lib.pa_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_out) and torch.equal(lse, want_lse), (H, Sq, Skv)
+        ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, :1].cpu(), k[:, :1].cpu(), v[:, :1].cpu())
+        assert (out[:, :1].float().cpu() - ref_out.float()).abs().max().item() <= 2e-2 + 2e-2 * ref_out.float().abs().max().item()
+        assert (lse[:, :1].cpu() - ref_lse).abs().max().item() <= 1e-3
+
+
 def test_noalloc_refuses_what_the_buffer_cannot_hold(cuda, tuning):
     lib = _lib.load()
     tuning("bm", 256)
