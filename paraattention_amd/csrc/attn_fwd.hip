@@ -882,18 +882,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
 //   barrier            K(j+1) and V(j) have landed; everybody is done with iteration j-1
 //   rare rescale of O  from the row maximum of S(j), taken one iteration earlier
 //   stage A  16 x { MFMA of S(j+1) = K(j+1) Q^T, its two key halves alternating ; one LDS-DMA issue
-//                   for K(j+2) / V(j+1) (first groups) ; refill of the consumed fragment slot ;
-//                   one slot of the softmax of S(j): scale, exp2, sum + pack of a score pair take
-//                   three consecutive slots }
-//   stage B  16 x { MFMA of O^T += V(j)^T P(j)^T ; refill ; the last softmax slots ; the row
-//                   maximum of S(j+1) }
+//                   for K(j+2) / V(j+1) (first groups) ; refill of the consumed fragment slot }
+//   six slots of the softmax of S(j) (a slot: scale of one score pair, exp2 of the pair before, row sum +
+//                   pack of the pair before that), which give the first PV MFMA its operand
+//   stage B  16 x { MFMA of O^T += V(j)^T P(j)^T ; refill ; one softmax slot under each of the first
+//                   twelve ; the row maximum of S(j+1) }
 //
-// That is the order of the source.  sched_barrier holds the MFMAs, the LDS reads and the tile copies
-// to it, but not the softmax arithmetic, which is pure: the compiler sinks it to its first use, so
-// the machine code runs stage A without VALU work, 22 of the 32 exponentials in front of the first
-// MFMA of stage B, the rest between its MFMAs and the row-sum additions behind the last one.  That
-// order is faster than the source's own (pinned with empty asm statements: -2 %) and than writing the
-// softmax as one block between the stages (-0.5 to -1.2 %), so the slots stay as they are.
+// sched_barrier holds the MFMAs, the LDS reads and the tile copies to that order, but not the softmax
+// arithmetic, which is pure; what holds it is the empty asm statement on the row sum in every slot.  Measured
+// against this arrangement: softmax slots under the MFMAs of stage A -2..-3.5 % (VALU work between the MFMAs of
+// the first GEMM costs more than it hides), the compiler's own placement (22 exponentials in front of stage B,
+// the row-sum additions behind the last MFMA) -0.7..-3 %, all of the softmax between the stages -0.5..-1.2 %,
+// its first slots right behind the barrier -1.5..-2.5 %.
 // Every iteration runs the same code: a tile that does not exist is fetched out of bounds (the
 // buffer descriptor returns zeros) and its scores are never used.
 // NW = 4 wavefronts (128 query rows, two workgroups per CU) or 8 (256 rows, one per CU: half the
@@ -1181,6 +1181,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       if (n >= 2 && n < 18) {
         const int j = n - 2;
         lsum += te[j & 1][0] + te[j & 1][1];
+        asm volatile("" : "+v"(lsum));  // the addition stays in its slot (left alone it sinks behind the last MFMA)
         (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
       }
       if (n >= 1 && n < 17) {
@@ -1206,7 +1207,6 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       if (g < IPW) dma_k1(par, n_nx2, g);                      // K(j+2) takes the buffer K(j) has left
       else if (g < 2 * IPW) dma_v1(par ^ 1, n_nxt, g - IPW);  // V(j+1) takes the buffer V(j-1) has left
       if (an) f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
-      if (ac) expo_slot(g);
       __builtin_amdgcn_sched_barrier(0);  // keep the groups in this order
     }
 #pragma unroll
@@ -1217,7 +1217,6 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       }
       if (ac) {
         f[g] = read_vt(tV, 0, g >> 2, g & 3);  // V(j), keys 0..31, takes the slot over
-        if (g < 4) expo_slot(8 + g);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1226,6 +1225,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    // The softmax of S(j) begins here, not under the MFMAs of stage A (VALU work between the MFMAs of the first GEMM
+    // costs more than it hides): the six slots that the first PV MFMA needs, then one slot under each of the next
+    // twelve PV MFMAs, each row-sum addition held in its slot.
+    if (ac) {
+#pragma unroll
+      for (int n = 0; n < 6; ++n) expo_slot(n);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     // ---- stage B ---------------------------------------------------------------------------------
     if constexpr (NW == 4) __builtin_amdgcn_s_setprio(1);
     __builtin_amdgcn_sched_barrier(0);
@@ -1249,7 +1256,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
         f[g] = read_vt(tV, 1, cc, db);  // keys 32..63
-        if (g < 6) expo_slot(12 + g);
+        expo_slot(6 + g);
         if (!BOUNDED && an) {
           if (g < 4) {
           } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
@@ -1267,6 +1274,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
       for (int db = 0; db < DB; ++db) {
         const int g = cc * 4 + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
+        if (g < 4) expo_slot(14 + g);
         if (!BOUNDED && an) {
           if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
         }
@@ -1441,7 +1449,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
 // O^T += V(j)^T P(j)^T (stage B), against the same 32 exponentials per lane as at head_dim 128, so
 // this kernel is bound by the VALU, not by the matrix cores.  The 8 fragments of K(j+1) fill the
 // ring at the top of an iteration; each stage-A MFMA frees a slot for one of the 8 fragments of
-// V(j); the 18 softmax slots sit two per group where the P half is needed soonest.
+// V(j); of the 18 softmax slots six sit between the stages (what the first PV MFMA needs) and three under
+// each of the first four PV MFMAs, held there by an empty asm statement on the row sum.
 // ---------------------------------------------------------------------------------------------
 constexpr int TILE64_BYTES = BN * 128;
 
@@ -1663,6 +1672,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
       if (n >= 2 && n < 18) {
         const int j = n - 2;
         lsum += te[j & 1][0] + te[j & 1][1];
+        asm volatile("" : "+v"(lsum));  // holds the slot's arithmetic where the source puts it
         (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
       }
       if (n >= 1 && n < 17) {
@@ -1678,7 +1688,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
     };
 #pragma unroll
     for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
-    // ---- stage A: S(j+1); slots 0..9 (P of keys 0..31 is complete when it ends) -----------------
+    // ---- stage A: S(j+1) ----------------------------------------------------------------------------
     if constexpr (NW == 4) __builtin_amdgcn_s_setprio(0);  // as in the head_dim 128 kernel
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
@@ -1687,18 +1697,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
       if (g < IPW) dma_k1(par, n_nx2, g);                      // K(j+2) takes the buffer K(j) has left
       else if (g < 2 * IPW) dma_v1(par ^ 1, n_nxt, g - IPW);  // V(j+1) takes the buffer V(j-1) has left
       f[g] = read_vt(tV, g >> 2, (g >> 1) & 1, g & 1);         // V(j) in the order stage B consumes it
-      if (g < 2) {
-        expo_slot(2 * g);
-        expo_slot(2 * g + 1);
-      } else {
-        expo_slot(g + 2);
-      }
       __builtin_amdgcn_sched_barrier(0);
     }
     if (v_nxt < BN || on_diagonal(n_nxt)) mask_tail(sn0, sn1, v_nxt, n_nxt);
     __builtin_amdgcn_sched_barrier(0);
 
-    // ---- stage B: O^T += V(j)^T P(j)^T; slots 10..17, then the row maximum of S(j+1) -------------
+    // the six softmax slots that the first PV MFMA needs (none under the MFMAs of stage A: measured -2 %)
+#pragma unroll
+    for (int n = 0; n < 6; ++n) expo_slot(n);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- stage B: O^T += V(j)^T P(j)^T; slots 6..17, three under each of the first four MFMAs, then the row
+    // maximum of S(j+1) ----------------------------------------------------------------------------
     if constexpr (NW == 4) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
@@ -1708,8 +1717,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
       for (int db = 0; db < DB; ++db) {
         const int g = 2 * cc + db;
         o[db] = T::mfma32(f[g], bfrag, o[db]);
-        expo_slot(10 + 2 * g);
-        expo_slot(11 + 2 * g);
+        expo_slot(6 + 3 * g);
+        expo_slot(7 + 3 * g);
+        expo_slot(8 + 3 * g);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
