@@ -431,6 +431,43 @@ def test_resident_workgroup_kernel(cuda, even, bound, tuning):
     assert lib.pa_attn_fwd_workspace_bytes(1, 24, 4608, 4608, 128, _lib.strides3(qf), _lib.strides3(qf)) == 0
 
 
+def test_resident_workgroups_with_a_short_workspace(cuda, tuning):
+    """pa_attn_fwd_lse_ws with less workspace than the plan asks for: the tail is cut into as many ranges as the
+    workspace holds (still more than its pieces), or, below that, left as whole pieces; with no workspace at all the
+    call runs as well.  Every variant against torch's CPU SDPA on sampled rows and against the full-workspace call."""
+    import ctypes
+
+    from paraattention_amd import _lib
+
+    lib = _lib.load()
+    tuning("bound", 0)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    B, H, D = 1, 2, 128
+    Sq, Skv = (cus // 2 + 20) * 256 - 31, 64 * 24 + 9  # one round and 40 pieces more
+    q, k, v = (t.to(cuda) for t in inputs.qkv(B, H, Sq, Skv, D, seed=8))
+    need = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, _lib.strides3(k), _lib.strides3(v))
+    per_range = 2 * 256 * 129 * 4
+    assert need > 100 * per_range, "meant to cut the 40 pieces of the tail into more than 100 ranges"
+    vp = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+    rows = torch.cat([torch.arange(0, 40), torch.arange(Sq - 300, Sq, 3)])
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, :, rows.to(cuda)].cpu(), k.cpu(), v.cpu())
+    results = []
+    for nbytes in (need, 100 * per_range + 77, 41 * per_range, 10 * per_range, 0):
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=cuda) if nbytes else None
+        out, lse = torch.empty_like(q), torch.empty((B, H, Sq), dtype=torch.float32, device=cuda)
+        rc = lib.pa_attn_fwd_lse_ws(vp(q), vp(k), vp(v), vp(out), vp(lse), 0, B, H, Sq, Skv, D, _lib.strides3(q),
+                                    _lib.strides3(k), _lib.strides3(v), _lib.strides3(out), 1.0 / math.sqrt(D), None, 0,
+                                    vp(ws), nbytes, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.pa_last_error()
+        torch.cuda.synchronize()
+        _check(out[:, :, rows.to(cuda)], lse[:, :, rows.to(cuda)], ref_out.float().numpy(), ref_lse.numpy(), f"workspace of {nbytes} bytes")
+        results.append((out, lse))
+    for out, lse in results[1:]:
+        assert (out.float() - results[0][0].float()).abs().max().item() <= 2e-2
+        assert (lse - results[0][1]).abs().max().item() <= 1e-4
+    assert torch.equal(results[3][0], results[4][0])  # too short for any cut and none at all: the same whole-piece plan
+
+
 @pytest.mark.parametrize("D,bm", [(128, "256"), (64, "128"), (64, "256")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_score_bound_variants(cuda, dtype, D, bm, tuning):
