@@ -1803,6 +1803,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                    // [2][64][256 B]
   char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
+  char* const sStage = (char*)smem + 4 * TILE_BYTES;  // [8 wavefronts][32 rows][256 B]: finished outputs on their way out
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -2043,7 +2044,35 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
     const Where w = where(kp, d.piece);
     const int my_row = w.row_begin + wave * 32 + l32;
     float* const acc_out = kp->acc_out;
-    if (my_row < w.row_end) {
+    if ((d.flags & FULL) && acc_out == nullptr) {
+      // A whole piece's output.  In the accumulator layout a lane holds 8-byte pieces of its row, 16 bytes apart,
+      // and a store instruction would touch 64 of them in 32 rows; staged through this wavefront's own 8 KB of
+      // LDS (16-byte chunks XOR-swizzled by the row, as the tiles are) the same data leaves as whole 256-byte rows,
+      // four per instruction.  Short pieces (cross-attention) store an output every few key tiles, and every
+      // store has to be through before the next barrier (one counter covers tile copies and stores).
+      char* const st = sStage + wave * 8192;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          u32x2 x;
+          x[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
+          x[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
+          *(u32x2*)(st + l32 * 256 + 16 * ((4 * db + a) ^ (l32 & 15)) + 8 * hh) = x;
+        }
+      uint16_t* const obase = (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h;
+      const int64_t os_s = kp->os_s;
+      const int row0 = w.row_begin + wave * 32;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int r = 4 * i + (lane >> 4), ch = lane & 15;
+        const u32x4 x = *(const u32x4*)(st + r * 256 + 16 * (ch ^ (r & 15)));
+        if (row0 + r < w.row_end) *(u32x4*)(obase + (int64_t)(row0 + r) * os_s + 8 * ch) = x;
+      }
+      float* const lse_out = kp->lse;
+      if (lse_out != nullptr && hh == 0 && my_row < w.row_end)
+        lse_out[((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row] = lse_nat;
+    } else if (my_row < w.row_end) {
       if (!(d.flags & FULL)) {  // a share of a piece: normalised fp32 partial + LSE into the workspace
         const int64_t wrow = (int64_t)(2 * wg + ((d.flags & MID) ? 0 : 1)) * 256 + (my_row - w.row_begin);
         float* wp = kp->ws_out + wrow * 128;
@@ -2092,19 +2121,6 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
             }
           }
         if (hh == 0) acc_lse[ridx] = lse_new;
-      } else {
-        uint16_t* op = (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h + (int64_t)my_row * kp->os_s;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            u32x2 x;
-            x[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
-            x[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
-            *(u32x2*)(op + 32 * db + 8 * a + 4 * hh) = x;
-          }
-        float* const lse_out = kp->lse;
-        if (lse_out != nullptr && hh == 0) lse_out[((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row] = lse_nat;
       }
     }
     // the next item starts from nothing
@@ -3129,7 +3145,7 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
 template <typename T>
 static int launch_stream(const AttnParams& p, hipStream_t stream) {
   if (p.out == nullptr && p.acc_out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
-  const size_t smem = 4 * TILE_BYTES;
+  const size_t smem = 4 * TILE_BYTES + 8 * 8192;  // two K and two V tiles, and a staging area for outputs
   static bool attr_done[PA_MAX_DEVICES][2] = {};  // benign race: the call is idempotent
   const int dev = current_device();
   for (int b = 0; b < 2; ++b) {
