@@ -96,9 +96,10 @@ PA_API int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* ou
  * scratch from torch's allocator; this library allocates nothing, so the caller
  * brings it.  With a workspace of at least pa_attn_fwd_workspace_bytes() bytes
  * (device memory, 16-byte aligned, contents irrelevant before and after) the
- * head_dim-128 kernel may compute the query tiles of the last, partly filled
- * round of workgroups in several key shares and fold them with the same
- * log-sum-exp merge as pa_merge_lse, which removes the idle tail of the launch.
+ * head_dim-128 kernels cut the query tiles that do not fill a round of the
+ * chip's compute units into ranges of key tiles, one per compute unit, and fold
+ * their partial results with the same log-sum-exp merge as pa_merge_lse, which
+ * removes the idle tail of the launch.
  * On launches of 2e12 flop and more the first 8 KB of the workspace hold a bound
  * of the scores, computed on the device from the largest row norms of q and k
  * (two small launches that read q and k once): where no score can leave
@@ -107,9 +108,10 @@ PA_API int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* ou
  * and always without a workspace, the variant with it.  Both are launched, and
  * the one the device-side flag does not select returns at once, so nothing is
  * read back by the host.
- * A null or short workspace is not an error: the call then runs as
- * pa_attn_fwd_lse does.  Results are the same to rounding.  Calls that share a
- * workspace must not overlap.
+ * A null or short workspace is not an error: the tail is then cut into as many
+ * ranges as the workspace holds, or not at all (as pa_attn_fwd_lse runs).
+ * Results are the same to rounding.  Calls that share a workspace must not
+ * overlap.
  */
 PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void* out, float* lse,
                        int dtype, int B, int H, int Sq, int Skv, int D,
@@ -225,7 +227,9 @@ PA_API size_t pa_attn_fwd_sweep_workspace_bytes(int B, int H, int Sq, int n_bloc
 
 /*
  * Bytes of workspace pa_attn_fwd_lse_ws and pa_attn_fwd_accumulate can use for this problem on the current
- * device (0: neither a key split nor a score bound would be used).  Depends on the device's CU count.
+ * device (0: neither partial results nor a score bound would be used): the larger of what a call with and a
+ * call without per-batch key counts / is_causal would take.  Depends on the device's CU count; at most about
+ * 68 MB on 256 compute units for a call without them (two fp32 partial results of 256 rows per compute unit).
  */
 PA_API size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
                                    const int64_t k_strides[3], const int64_t v_strides[3]);
