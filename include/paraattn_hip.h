@@ -100,7 +100,7 @@ PA_API int pa_attn_fwd_lse(const void* q, const void* k, const void* v, void* ou
  * chip's compute units into ranges of key tiles, one per compute unit, and fold
  * their partial results with the same log-sum-exp merge as pa_merge_lse, which
  * removes the idle tail of the launch.
- * On launches of 2e12 flop and more the first 8 KB of the workspace hold a bound
+ * On launches of 1e12 flop and more the first 8 KB of the workspace hold a bound
  * of the scores, computed on the device from the largest row norms of q and k
  * (two small launches that read q and k once): where no score can leave
  * [-60, 60] in the log2 domain (models that normalise q and k sit near 16) the
