@@ -10,17 +10,20 @@ from oracle import inputs
 pytestmark = pytest.mark.gpu
 
 
-def _eager(q, kb, vb, prev, cur, key_mask):
+def _eager(q, kb, vb, prev, cur, key_mask, block_mask):
     out, lse = torch.ops.para_attn.attention_forward_with_lse(q, kb[0], vb[0])
     # masked calls: whether the key mask is a prefix is decided on the device, inside the captured work
     mo, ml = torch.ops.para_attn.attention_forward_with_lse(q, kb[0], vb[0], key_mask)
     so = torch.ops.para_attn.attention_forward_sparse_kv(q, kb[0], vb[0], key_mask.expand(-1, -1, q.shape[2], -1))
     ro, rl = paraattention_amd.ring_sweep(q, kb, vb, fused=True)
     uo, ul = paraattention_amd.ring_sweep(q, kb, vb, fused=False)
+    wo, wl = paraattention_amd.ring_sweep(q, kb, vb)  # all blocks in one launch
+    # block-sparse with the ranges extracted inside the captured work
+    bo, bl = torch.ops.para_attn.attention_forward_block_sparse(q[:, :, :1024], kb[0][:, :, :2560], vb[0][:, :, :2560], block_mask)
     ratio = torch.ops.para_attn.fbcache_residual_diff(prev, cur)
     applied = torch.ops.para_attn.fbcache_apply_residual(prev, cur)
     tv = torch.ops.para_attn.taylorseer_value([cur, prev], 2, prev)
-    return [out, lse, ro, rl, uo, ul, ratio, applied, tv, mo, ml, so]
+    return [out, lse, ro, rl, uo, ul, ratio, applied, tv, mo, ml, so, wo, wl, bo, bl]
 
 
 def test_graph_replays_match_eager(cuda):
@@ -33,18 +36,19 @@ def test_graph_replays_match_eager(cuda):
     vb = [t.contiguous().to(cuda) for t in v.split(2600, 2)]
     prev, cur = (t.to(cuda) for t in inputs.fbcache_pair((1, 700, 512), seed=2))
     key_mask = (torch.arange(2600)[None, None, None, :] < 2000).to(cuda)  # a prefix at capture time
-    _eager(q, kb, vb, prev, cur, key_mask)  # warm-up outside capture (library load, function attributes)
+    block_mask = (torch.rand(8, 20, generator=torch.Generator().manual_seed(3)) < 0.5).to(cuda)  # 128-row x 128-key blocks
+    _eager(q, kb, vb, prev, cur, key_mask, block_mask)  # warm-up outside capture (library load, function attributes)
     key_mask[..., 5] = False
-    _eager(q, kb, vb, prev, cur, key_mask)  # and the per-score kernel's
+    _eager(q, kb, vb, prev, cur, key_mask, block_mask)  # and the per-score kernel's
     key_mask[..., 5] = True
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
-        _eager(q, kb, vb, prev, cur, key_mask)
+        _eager(q, kb, vb, prev, cur, key_mask, block_mask)
         torch.cuda.synchronize()
         with torch.cuda.graph(graph, stream=side):
-            captured = _eager(q, kb, vb, prev, cur, key_mask)
+            captured = _eager(q, kb, vb, prev, cur, key_mask, block_mask)
     torch.cuda.synchronize()
     g = torch.Generator().manual_seed(5)
     for rep in range(4):
@@ -57,7 +61,7 @@ def test_graph_replays_match_eager(cuda):
         graph.replay()
         torch.cuda.synchronize()
         got = [t.clone() for t in captured]
-        want = _eager(q, kb, vb, prev, cur, key_mask)
+        want = _eager(q, kb, vb, prev, cur, key_mask, block_mask)
         torch.cuda.synchronize()
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), f"replay {rep}: output {i} differs from the eager run"
