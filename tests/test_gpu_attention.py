@@ -536,6 +536,23 @@ def test_causal_reference_test_shape(cuda, dtype, D):
     _check(out[:, hs], lse[:, hs], ref_out.numpy(), ref_lse.numpy(), f"causal 4096 {dtype} D={D}")
 
 
+def test_causal_long_sequence_sampled_rows(cuda):
+    """is_causal at a length where the launch has many rounds of workgroups of unequal length (started longest
+    first) and most tiles lie below the diagonal: sampled rows against torch's CPU SDPA over each row's own key
+    prefix, every row's LSE against the count of keys it sees for zero queries."""
+    B, H, S, D = 1, 2, 20000 + 37, 128
+    q, k, v = inputs.qkv(B, H, S, S, D, seed=12)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, is_causal=True)
+    g = torch.Generator().manual_seed(4)
+    for r in [0, 1, 63, 64, 255, 256, S - 1] + torch.randint(0, S, (10,), generator=g).tolist():
+        ro, rl = oattn.sdpa_lse_torch_cpu(q[:, :, r : r + 1], k[:, :, : r + 1], v[:, :, : r + 1])
+        _check(out[:, :, r : r + 1], lse[:, :, r : r + 1], ro.float().numpy(), rl.numpy(), f"causal row {r}")
+    _, lse0 = torch.ops.para_attn.attention_forward_with_lse(torch.zeros_like(qd), kd, vd, is_causal=True)
+    want = torch.log(torch.arange(1, S + 1, dtype=torch.float64))[None, None, :].expand(B, H, S)
+    assert (lse0.cpu().double() - want).abs().max().item() <= 1e-3
+
+
 def test_causal_argument_rules(cuda):
     q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 32, 32, 128))
     mask = torch.ones(1, 1, 1, 32, dtype=torch.bool, device=cuda)
