@@ -53,9 +53,35 @@ def _kernel_ready(t):
     return t
 
 
+def _out_like(query):
+    """The attention output for ``query``: the query's own memory layout (a [B,S,H,D]-memory view stays one, so the
+    caller's transpose back is free) whenever the kernels can write it -- unit head_dim stride, 16-byte aligned rows
+    -- and contiguous otherwise.  Reads sizes and strides only, so the fake implementations allocate through it
+    too and a compiled graph is planned against the strides the kernel really writes."""
+    out = torch.empty_like(query)
+    if out.stride(-1) != 1 or any(out.shape[d] > 1 and out.stride(d) % 8 for d in range(out.ndim - 1)):
+        out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+    return out
+
+
+def _lse_like(query):
+    B, H, Sq, _ = query.shape
+    return torch.empty((B, H, Sq), dtype=torch.float32, device=query.device)
+
+
+def _same_device(ref, **operands):
+    """The kernels take raw pointers, so an operand on another device (a CPU mask beside GPU activations) must stop
+    here with an error, as it does in the aten ops the reference calls, and not at a memory fault on the GPU.
+    Every function below that hands a tensor's pointer to the library runs its tensors through this first."""
+    for name, t in operands.items():
+        if t is not None and t.device != ref.device:
+            raise ValueError(f"{name} is on {t.device} but must be on {ref.device}: all operands must share one device")
+
+
 def _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask=None, causal_ok=False):
     if query.ndim != 4 or key.ndim != 4 or value.ndim != 4:
         raise ValueError("query, key and value must be 4-D [batch, heads, seq, head_dim]")
+    _same_device(query, key=key, value=value, attn_mask=attn_mask)
     if dropout_p != 0.0:
         raise NotImplementedError("dropout_p > 0 is not supported (the reference's hot path is inference only)")
     if is_causal and not causal_ok:
@@ -76,11 +102,10 @@ def _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask=None, ca
 def _dense_forward(query, key, value, scale, want_lse, kv_len=None, is_causal=False):
     B, H, Sq, D = query.shape
     Skv = key.shape[2]
+    _same_device(query, key=key, value=value, kv_len=kv_len)
     q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
-    out = torch.empty_like(q)
-    if out.stride(-1) != 1:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    out = _out_like(query)
+    lse = _lse_like(query) if want_lse else None
     if scale is None:
         scale = 1.0 / math.sqrt(D)
     lib = _lib.load()
@@ -111,6 +136,7 @@ def _accumulate_forward(acc_out, acc_lse, query, key, value, scale, first, final
         raise ValueError("accumulator shapes must be [B,H,Sq,D] and [B,H,Sq]")
     if not acc_out.is_contiguous() or not acc_lse.is_contiguous():
         raise ValueError("accumulators must be contiguous")
+    _same_device(query, key=key, value=value, acc_out=acc_out, acc_lse=acc_lse)
     q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device) if final else None
     if scale is None:
@@ -164,12 +190,11 @@ def _masked_forward(query, key, value, attn_mask, scale, want_lse, is_causal=Fal
         return _dense_forward(query, key, value, scale, want_lse, is_causal=is_causal)
     B, H, Sq, D = query.shape
     Skv = key.shape[2]
+    _same_device(query, key=key, value=value, attn_mask=attn_mask)
     mask, kind, mstrides = _broadcast_mask(attn_mask, B, H, Sq, Skv, query.dtype)
     q, k, v = _kernel_ready(query), _kernel_ready(key), _kernel_ready(value)
-    out = torch.empty_like(q)
-    if out.stride(-1) != 1:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    out = _out_like(query)
+    lse = _lse_like(query) if want_lse else None
     if scale is None:
         scale = 1.0 / math.sqrt(D)
     lib = _lib.load()
@@ -209,10 +234,7 @@ def attention_forward_with_lse(
 
 @torch.library.register_fake("para_attn::attention_forward_with_lse")
 def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
-    B, H, Sq, _ = query.shape
-    out = query.new_empty((B, H, Sq, value.shape[-1]))
-    lse = query.new_empty((B, H, Sq), dtype=torch.float32)
-    return out, lse
+    return _out_like(query), _lse_like(query)
 
 
 @torch.library.custom_op("para_attn::attention_forward", mutates_args=(), device_types=("cuda",))
@@ -234,8 +256,7 @@ def attention_forward(
 
 @torch.library.register_fake("para_attn::attention_forward")
 def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
-    B, H, Sq, _ = query.shape
-    return query.new_empty((B, H, Sq, value.shape[-1]))
+    return _out_like(query)
 
 
 @torch.library.custom_op("para_attn::attention_forward_sparse_kv", mutates_args=(), device_types=("cuda",))
@@ -256,7 +277,7 @@ def attention_forward_sparse_kv(
     excludes is_causal (:270).  A prefix mask (valid text length) costs nothing:
     the kernel just stops at the per-batch key count.
     """
-    _check_sdpa_args(query, key, value, dropout_p, is_causal)
+    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask)
     if attn_mask is None:
         return _dense_forward(query, key, value, scale, False)[0]
     if attn_mask.dtype != torch.bool:
@@ -274,8 +295,7 @@ def attention_forward_sparse_kv(
 
 @torch.library.register_fake("para_attn::attention_forward_sparse_kv")
 def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
-    B, H, Sq, _ = query.shape
-    return query.new_empty((B, H, Sq, value.shape[-1]))
+    return _out_like(query)
 
 
 # ---------------------------------------------------------------------------------
@@ -295,6 +315,7 @@ def _merge_launch(acc_out, acc_lse, blk_out, blk_lse, out, lse_out):
 
 
 def _check_merge_args(acc_out, acc_lse, blk_out, blk_lse):
+    _same_device(acc_out, acc_lse=acc_lse, blk_out=blk_out, blk_lse=blk_lse)
     if acc_out.shape != blk_out.shape:
         raise ValueError(f"partial outputs differ in shape: {tuple(acc_out.shape)} vs {tuple(blk_out.shape)}")
     rows = acc_out.numel() // max(acc_out.shape[-1], 1)
@@ -433,10 +454,8 @@ def attention_forward_sweep(
         vs = [t.contiguous() for t in vs]
     blk = ks[0].shape[2]
     q = _kernel_ready(query)
-    out = torch.empty_like(q)
-    if out.stride(-1) != 1:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    out = _out_like(query)
+    lse = _lse_like(query)
     if scale is None:
         scale = 1.0 / math.sqrt(D)
     lib = _lib.load()
@@ -454,8 +473,7 @@ def attention_forward_sweep(
 
 @torch.library.register_fake("para_attn::attention_forward_sweep")
 def _(query, key_blocks, value_blocks, *, scale=None):
-    B, H, Sq, _ = query.shape
-    return query.new_empty(query.shape), query.new_empty((B, H, Sq), dtype=torch.float32)
+    return _out_like(query), _lse_like(query)
 
 
 # ---------------------------------------------------------------------------------
@@ -485,12 +503,7 @@ def _sparse_geometry(query, key, block_mask_shape, q_lo, q_hi, kv_lo, kv_hi):
 
 
 def _sparse_outputs(query):
-    q = _kernel_ready(query)
-    out = torch.empty_like(q)
-    if out.stride(-1) != 1:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    B, H, Sq, _ = q.shape
-    return q, out, torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    return _kernel_ready(query), _out_like(query), _lse_like(query)
 
 
 @torch.library.custom_op("para_attn::attention_forward_block_sparse", mutates_args=(), device_types=("cuda",))
@@ -520,6 +533,7 @@ def attention_forward_block_sparse(
     Skv = key.shape[2]
     if block_mask.dtype != torch.bool:
         raise ValueError("block_mask must be boolean")
+    _same_device(query, block_mask=block_mask)
     if block_mask.ndim == 2:
         block_mask = block_mask.unsqueeze(0)
     Hm, nQ, nK, q_lo, q_hi, kv_lo, kv_hi, q_block, kv_block = _sparse_geometry(query, key, block_mask.shape, q_lo, q_hi, kv_lo, kv_hi)
@@ -544,8 +558,13 @@ def attention_forward_block_sparse(
 
 @torch.library.register_fake("para_attn::attention_forward_block_sparse")
 def _(query, key, value, block_mask, q_lo=0, q_hi=-1, kv_lo=0, kv_hi=-1, *, scale=None):
-    B, H, Sq, _ = query.shape
-    return query.new_empty((B, H, Sq, value.shape[-1])), query.new_empty((B, H, Sq), dtype=torch.float32)
+    return _out_like(query), _lse_like(query)
+
+
+def _runs_words(Hm, nQ, nK):
+    """Length in int32 words of the key-range buffer of a [Hm,nQ,nK] mask: the library's own figure (host
+    arithmetic, no device call), so the op and its fake implementation cannot disagree."""
+    return (_lib.load().pa_blocksparse_workspace_bytes(Hm, nQ, nK) + 3) // 4
 
 
 @torch.library.custom_op("para_attn::block_sparse_key_runs", mutates_args=(), device_types=("cuda",))
@@ -566,8 +585,8 @@ def block_sparse_key_runs(block_mask: torch.Tensor, seq_kv: int, kv_lo: int = 0,
         raise ValueError("block_mask must divide a non-empty sparse key/value range inside the keys")
     kv_block = (kv_hi - kv_lo) // nK
     lib = _lib.load()
-    ws_bytes = lib.pa_blocksparse_workspace_bytes(Hm, nQ, nK)
-    ws = torch.zeros((ws_bytes + 3) // 4, dtype=torch.int32, device=block_mask.device)
+    ws = torch.zeros(_runs_words(Hm, nQ, nK), dtype=torch.int32, device=block_mask.device)
+    ws_bytes = ws.numel() * 4
     mask_u8 = block_mask.contiguous().view(torch.uint8)
     with torch.cuda.device(block_mask.device):
         rc = lib.pa_blocksparse_build_runs(
@@ -580,8 +599,7 @@ def block_sparse_key_runs(block_mask: torch.Tensor, seq_kv: int, kv_lo: int = 0,
 @torch.library.register_fake("para_attn::block_sparse_key_runs")
 def _(block_mask, seq_kv, kv_lo=0, kv_hi=-1):
     Hm, nQ, nK = block_mask.shape if block_mask.ndim == 3 else (1, *block_mask.shape)
-    nseg, cap = nQ + 2, nK // 2 + 3
-    return block_mask.new_empty((Hm * nseg + Hm * nseg * cap * 2,), dtype=torch.int32)
+    return block_mask.new_empty((_runs_words(Hm, nQ, nK),), dtype=torch.int32)
 
 
 @torch.library.custom_op("para_attn::attention_forward_block_sparse_runs", mutates_args=(), device_types=("cuda",))
@@ -626,8 +644,7 @@ def attention_forward_block_sparse_runs(
 
 @torch.library.register_fake("para_attn::attention_forward_block_sparse_runs")
 def _(query, key, value, runs, mask_heads, n_q, n_k, q_lo=0, q_hi=-1, *, scale=None):
-    B, H, Sq, _ = query.shape
-    return query.new_empty((B, H, Sq, value.shape[-1])), query.new_empty((B, H, Sq), dtype=torch.float32)
+    return _out_like(query), _lse_like(query)
 
 
 def block_sparse_runs(block_mask, Skv, kv_lo=0, kv_hi=-1):
@@ -700,6 +717,7 @@ def fbcache_residual_diff(prev: torch.Tensor, cur: torch.Tensor) -> torch.Tensor
         raise NotImplementedError(f"dtypes {prev.dtype}/{cur.dtype} not supported")
     if prev.numel() == 0:
         raise ValueError("mean of an empty tensor")
+    _same_device(prev, cur=cur)
     pr, cr = _as_rows(prev), _as_rows(cur)
     if pr is None:
         prev = prev.contiguous()
@@ -735,6 +753,7 @@ def fbcache_first_residual_diff(
         raise ValueError("hidden and hidden0 must share shape and a supported dtype")
     if prev is not None and (prev.shape != hidden.shape or prev.dtype != hidden.dtype):
         raise ValueError("prev must match hidden in shape and dtype")
+    _same_device(hidden, hidden0=hidden0, prev=prev)
     h, h0 = hidden.contiguous(), hidden0.contiguous()
     pv = prev.contiguous() if prev is not None else None
     resid = torch.empty(h.shape, dtype=h.dtype, device=h.device)
@@ -760,6 +779,7 @@ def fbcache_apply_residual(residual: torch.Tensor, hidden: torch.Tensor) -> torc
     """``residual + hidden``, contiguous (src/para_attn/first_block_cache/utils.py:237-259)."""
     if residual.shape != hidden.shape or residual.dtype != hidden.dtype or hidden.dtype not in _DTYPE_CODE:
         raise ValueError("residual and hidden must share shape and a supported dtype")
+    _same_device(hidden, residual=residual)
     r, h = residual.contiguous(), hidden.contiguous()
     out = torch.empty(h.shape, dtype=h.dtype, device=h.device)
     lib = _lib.load()
@@ -812,7 +832,7 @@ def taylorseer_derivatives(y: torch.Tensor, prev: List[torch.Tensor], window: fl
 
 @torch.library.register_fake("para_attn::taylorseer_derivatives")
 def _(y, prev, window):
-    return [torch.empty_like(y) for _ in prev]
+    return [y.new_empty(y.shape) for _ in prev]
 
 
 @torch.library.custom_op("para_attn::taylorseer_value", mutates_args=(), device_types=("cuda",))
@@ -841,4 +861,4 @@ def taylorseer_value(derivs: List[torch.Tensor], elapsed: int, hidden: Optional[
 
 @torch.library.register_fake("para_attn::taylorseer_value")
 def _(derivs, elapsed, hidden=None):
-    return torch.empty_like(derivs[0])
+    return derivs[0].new_empty(derivs[0].shape)

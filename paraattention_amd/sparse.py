@@ -2,11 +2,15 @@
 (src/para_attn/sparse_attn.py:285-311, 643-693): same arguments, one kernel
 launch instead of a Python loop of SDPA calls and merges.
 """
+import weakref
+
 import torch
 import torch.nn.functional as F
 
 from . import ops
 from .interface import _SdpaMode
+
+_RUNS_CACHE_ENTRIES = 4
 
 
 def struct_sparse_attn_func(
@@ -56,14 +60,22 @@ def struct_sparse_attn_func(
         mask = sparse_mask.to(device=query.device, dtype=torch.bool)
         out, _ = ops.attention_forward_block_sparse(query, key, value, mask, q_lo, q_hi, kv_lo, kv_hi, scale=scale)
         return out
-    # the mask's content is identified by the tensor and its version counter (in-place edits bump it)
-    tag = (id(sparse_mask), sparse_mask._version, query.device, s_kv, kv_lo, kv_hi)
-    runs = runs_cache.get(tag)
-    if runs is None:
+    # An entry serves one (key length, sparse key range, device); it remembers which mask it was built from by a
+    # weak reference (an id() alone could be a later tensor at a freed one's address) and by the mask's version
+    # counter (in-place edits bump it).  A few entries are kept, so a model that sends two or three key lengths
+    # through the mode in one step scans the mask once for each and not once per call.
+    tag = (query.device, s_kv, kv_lo, kv_hi)
+    entry = runs_cache.get(tag)
+    if entry is not None and (entry[0]() is not sparse_mask or entry[1] != sparse_mask._version):
+        entry = None
+    if entry is None:
         mask = sparse_mask.to(device=query.device, dtype=torch.bool)
         runs = ops.block_sparse_key_runs(mask, s_kv, kv_lo, kv_hi)
-        runs_cache.clear()  # one mask, one key length at a time: no pile of stale entries
-        runs_cache[tag] = runs
+        runs_cache.pop(tag, None)
+        while len(runs_cache) >= _RUNS_CACHE_ENTRIES:
+            runs_cache.pop(next(iter(runs_cache)))  # oldest first
+        runs_cache[tag] = entry = (weakref.ref(sparse_mask), sparse_mask._version, runs)
+    runs = entry[2]
     shape = (1, *sparse_mask.shape) if sparse_mask.ndim == 2 else tuple(sparse_mask.shape)
     out, _ = ops.attention_forward_block_sparse_runs(query, key, value, runs, shape[0], shape[1], shape[2], q_lo, q_hi, scale=scale)
     return out

@@ -52,6 +52,89 @@ def test_fake_impls_give_reference_contract():
         assert r.shape == () and r.dtype == torch.bfloat16
 
 
+def test_fake_outputs_keep_the_query_layout():
+    """The real ops write the output in the query's memory layout (ops._out_like); the fakes must describe the same
+    strides or a compiled consumer is planned against the wrong ones.  The GPU suite compares fake and real with
+    torch.library.opcheck; here the rule itself is pinned without a device."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    ns = torch.ops.para_attn
+    with FakeTensorMode():
+        bshd = torch.empty(2, 200, 3, 128, dtype=torch.bfloat16, device="cuda").transpose(1, 2)
+        assert bshd.stride() == (76800, 128, 384, 1)
+        bm = torch.empty(3, 2, 4, dtype=torch.bool, device="cuda")
+        runs = ns.block_sparse_key_runs(bm, 200)
+        outs = [
+            ns.attention_forward_with_lse(bshd, bshd, bshd)[0],
+            ns.attention_forward(bshd, bshd, bshd),
+            ns.attention_forward_sparse_kv(bshd, bshd, bshd),
+            ns.attention_forward_sweep(bshd, [bshd], [bshd])[0],
+            ns.attention_forward_block_sparse(bshd, bshd, bshd, bm)[0],
+            ns.attention_forward_block_sparse_runs(bshd, bshd, bshd, runs, 3, 2, 4)[0],
+        ]
+        for o in outs:
+            assert o.shape == bshd.shape and o.stride() == bshd.stride()
+        assert ns.attention_forward_with_lse(bshd, bshd, bshd)[1].stride() == (600, 200, 1)
+        # rows the kernels cannot write in place (row stride not a multiple of 8 elements; head_dim not innermost)
+        ragged = torch.empty(2, 3, 200, 132, dtype=torch.bfloat16, device="cuda")[..., :128]
+        assert ns.attention_forward(ragged, ragged, ragged).is_contiguous()
+        dfirst = torch.empty(2, 3, 128, 200, dtype=torch.bfloat16, device="cuda").transpose(2, 3)
+        assert ns.attention_forward(dfirst, dfirst, dfirst).is_contiguous()
+        # the key-range buffer: the library's own size for the mask geometry, single and paired layouts
+        lib = paraattention_amd._lib.load()
+        for hm, nq, nk in ((1, 2, 64), (3, 2, 4), (24, 256, 256)):
+            words = ns.block_sparse_key_runs(torch.empty(hm, nq, nk, dtype=torch.bool, device="cuda"), nk * 128).numel()
+            assert words * 4 >= lib.pa_blocksparse_workspace_bytes(hm, nq, nk) > (words - 1) * 4
+
+
+def test_operands_of_another_device_stop_before_any_launch():
+    """The op bodies, called directly with the query on one device ("meta": no memory, so nothing can be launched
+    from it) and another operand on the CPU: every one of them raises the device error first.  A CPU mask beside
+    GPU activations reaches the GPU implementation (the dispatcher picks it for the mixed call), where its pointer
+    would be read by a kernel."""
+    bf = torch.bfloat16
+    q = torch.empty(2, 2, 64, 128, dtype=bf, device="meta")
+    cq = torch.empty(2, 2, 64, 128, dtype=bf)
+    keep = torch.ones(2, 1, 1, 64, dtype=torch.bool)
+    lse, clse = torch.empty(2, 2, 64, device="meta"), torch.empty(2, 2, 64)
+    acc, cacc = torch.empty(2, 2, 64, 128, device="meta"), torch.empty(2, 2, 64, 128)
+    bm = torch.ones(2, 2, dtype=torch.bool)
+    h, ch = torch.empty(4, 64, dtype=bf, device="meta"), torch.empty(4, 64, dtype=bf)
+    calls = [
+        (ops.attention_forward_with_lse, (q, q, q, keep)),
+        (ops.attention_forward_with_lse, (q, q, q, keep.float())),
+        (ops.attention_forward_with_lse, (q, cq, q)),
+        (ops.attention_forward_with_lse, (q, q, cq)),
+        (ops.attention_forward, (q, q, q, keep)),
+        (ops.attention_forward, (q, cq, cq)),
+        (ops.attention_forward_sparse_kv, (q, q, q, keep)),
+        (ops.attention_forward_sparse_kv, (q, q, cq)),
+        (ops.merge_attention_lse, (acc, clse, q, lse)),
+        (ops.merge_attention_lse, (acc, lse, cq, lse)),
+        (ops.merge_attention_lse, (acc, lse, q, clse)),
+        (ops.merge_attention_lse_, (acc, lse, cq, lse)),
+        (ops.attention_forward_accumulate_, (cacc, lse, q, q, q)),
+        (ops.attention_forward_accumulate_, (acc, clse, q, q, q)),
+        (ops.attention_forward_accumulate_, (acc, lse, q, cq, q)),
+        (ops.attention_forward_accumulate_final, (acc, clse, q, q, q)),
+        (ops.attention_forward_sweep, (q, [q, cq], [q, q])),
+        (ops.attention_forward_sweep, (q, [q, q], [cq, q])),
+        (ops.attention_forward_block_sparse, (q, q, q, bm)),
+        (ops.attention_forward_block_sparse, (q, cq, q, bm.to("meta"))),
+        (ops.attention_forward_block_sparse_runs, (q, q, q, torch.zeros(64, dtype=torch.int32), 1, 2, 2)),
+        (ops.fbcache_residual_diff, (h, ch)),
+        (ops.fbcache_first_residual_diff, (h, ch)),
+        (ops.fbcache_first_residual_diff, (h, h, ch)),
+        (ops.fbcache_apply_residual, (ch, h)),
+        (ops.taylorseer_derivatives, (h, [h, ch], 2.0)),
+        (ops.taylorseer_value, ([h, ch], 2)),
+        (ops.taylorseer_value, ([h, h], 2, ch)),
+    ]
+    for op, args in calls:
+        with pytest.raises(ValueError, match="device"):
+            op._init_fn(*args)
+
+
 def test_cpu_tensors_are_refused_not_emulated():
     # the reference asserts "Must be CUDA tensors" (src/para_attn/ops/__init__.py:123); here the dispatcher refuses
     q = torch.randn(1, 1, 16, 128).bfloat16()
