@@ -19,7 +19,7 @@ the gap), so the defaults warm every loop up for that long (30 calls of the head
 memory-side cache cannot hold a working set from one call to the next; a sample of rows of the last
 timed output of every attention shape is compared with torch's CPU SDPA (``checked``).
 
-``--only {attn,merge,fbcache,taylorseer,sparse,ring,flux,wan,shapes,copy}`` runs a single loop (what
+``--only {attn,merge,fbcache,taylorseer,sparse,ring,flux,wan,shapes,copy,yardsticks}`` runs a single loop (what
 the rocprofv3 summaries under profiles/ were taken with).
 """
 import argparse
@@ -90,15 +90,18 @@ def _mfma(workload, flops, t, **more):
             "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4), **more}
 
 
-def _check_rows(out, lse, q, k, v, heads, rows, what):
+def _check_rows(out, lse, q, k, v, heads, rows, what, causal=False):
     """Compares sampled query rows of a timed call's output with torch's CPU SDPA on the same bits (the routine
-    the oracle is pinned to); raises if they differ by more than the parity tolerance, else returns True."""
+    the oracle is pinned to); raises if they differ by more than the parity tolerance, else returns True.
+    ``causal``: the sampled rows see keys 0..row only (is_causal of the full problem, as a mask for the sample)."""
     import torch
 
     from oracle import attention as oattn
 
     rows = torch.as_tensor(rows)
-    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, heads][:, :, rows].contiguous(), k[:, heads].contiguous(), v[:, heads].contiguous())
+    keep = (torch.arange(k.shape[2])[None, :] <= rows[:, None])[None, None] if causal else None
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, heads][:, :, rows].contiguous(), k[:, heads].contiguous(), v[:, heads].contiguous(),
+                                                attn_mask=keep)
     got = out[:, heads][:, :, rows.to(out.device)].float().cpu()
     err = (got - ref_out.float()).abs()
     if not bool((err <= 2e-2 + 2e-2 * ref_out.float().abs()).all()):
@@ -140,32 +143,42 @@ def bench_attn(dev, steps, warmup):
     return (q, k, v), 4.0 * B * H * S * S * D, t, checked
 
 
-def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=(0,), traffic=None):
+def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=(0,), traffic=None, causal=False, sets=1):
+    """One dense shape: timed, then sampled rows of the last timed output checked against torch's CPU SDPA.
+    ``sets`` > 1: the calls rotate over that many copies of q, k, v at different addresses, so that a working set
+    smaller than the 256 MB memory-side cache is not served from it call after call (in a model every call brings
+    other tensors)."""
     import torch
 
     from oracle import inputs
 
     q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=seed)
-    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    bufs = [(q.to(dev), k.to(dev), v.to(dev)) for _ in range(sets)]
     op = torch.ops.para_attn.attention_forward_with_lse
     last = {}
 
     def call(i):
-        last["out"], last["lse"] = op(qd, kd, vd)
+        qd, kd, vd = bufs[i % sets]
+        last["out"], last["lse"] = op(qd, kd, vd, is_causal=causal)
 
     t = _time_calls(call, steps, warmup)
     heads = sorted(set(list(check_heads) + [H - 1]))
-    checked = _check_rows(last["out"], last["lse"], q, k, v, heads, _sample_rows(Sq), name)
-    flops = 4.0 * B * H * Sq * Skv * D
+    checked = _check_rows(last["out"], last["lse"], q, k, v, heads, _sample_rows(Sq), name, causal=causal)
+    flops = 4.0 * B * H * Sq * Skv * D * (0.5 if causal else 1.0)  # causal: the kept half (Sq == Skv)
     nbytes = 2.0 * B * H * D * (2 * Sq + 2 * Skv) + 4.0 * B * H * Sq
     gbs = nbytes / (t["median"] * 1e-3) / 1e9
     more = {"traffic": TRAFFIC[traffic], "traffic_source": TRAFFIC_SOURCE} if traffic else {}
-    return _mfma(f"{name}: attention_forward_with_lse q [{B},{H},{Sq},{D}] k,v [{B},{H},{Skv},{D}] bf16", flops, t,
+    if sets > 1:
+        more["buffer_sets"] = sets
+    what = "attention_forward_with_lse" + (" is_causal" if causal else "")
+    return _mfma(f"{name}: {what} q [{B},{H},{Sq},{D}] k,v [{B},{H},{Skv},{D}] bf16", flops, t,
                  bytes=nbytes, gbs=round(gbs, 1), frac_hbm=round(gbs / PEAK_HBM_GBS, 4), checked=checked, **more)
 
 
 def bench_flux(dev, steps=50, warmup=100):
-    return _dense_case(dev, "FLUX joint attention", 1, 24, 4608, 4608, 128, steps, warmup, seed=0, traffic="flux")
+    """FLUX-dev joint attention.  q, k, v and the output are 113 MB together, less than the memory-side cache: four
+    sets of inputs are rotated."""
+    return _dense_case(dev, "FLUX joint attention", 1, 24, 4608, 4608, 128, steps, warmup, seed=0, traffic="flux", sets=4)
 
 
 def bench_wan(dev, steps=10, warmup=10):
@@ -212,26 +225,14 @@ def bench_ring(dev, steps=6, warmup=3):
     return out
 
 
-def bench_shapes(dev, steps=10, warmup=3):
-    """Further dense shapes (not part of the default run): the headline shape with is_causal and a head_dim 64 shape."""
-    import torch
-
-    op = torch.ops.para_attn.attention_forward_with_lse
-    rows = []
-    cases = [
-        ("headline shape, is_causal", 1, 3, 119056, 119056, 128, True),
-        ("head_dim 64 (CogVideoX-like)", 1, 48, 17776, 17776, 64, False),
-    ]
-    for name, B, H, Sq, Skv, D, causal in cases:
-        g = torch.Generator().manual_seed(3)
-        q = torch.randn(B, H, Sq, D, generator=g).bfloat16().to(dev)
-        k = torch.randn(B, H, Skv, D, generator=g).bfloat16().to(dev)
-        v = torch.randn(B, H, Skv, D, generator=g).bfloat16().to(dev)
-        t = _time_calls(lambda i: op(q, k, v, is_causal=causal), steps, warmup)
-        flops = 4.0 * B * H * Sq * Skv * D * (0.5 if causal else 1.0)  # causal: the kept half (Sq == Skv)
-        rows.append(_mfma(f"{name}: q [{B},{H},{Sq},{D}] k,v [{B},{H},{Skv},{D}] bf16", flops, t))
-        del q, k, v
-    return rows
+def bench_shapes(dev, steps=10, warmup=5):
+    """Two further dense shapes: the headline shape with is_causal (flops of the kept half) and a head_dim 64 shape."""
+    return {
+        "headline_shape_causal": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=5,
+                                             check_heads=(0, 1), causal=True),
+        "head_dim_64": _dense_case(dev, "head_dim 64 (CogVideoX-like)", 1, 48, 17776, 17776, 64, steps, warmup, seed=6,
+                                   check_heads=(0, 23)),
+    }
 
 
 def bench_sparse(dev, steps=10, warmup=10):
@@ -348,6 +349,30 @@ def bench_copy(dev, steps=10, warmup=2):
     return r
 
 
+def bench_yardsticks(dev, steps=30, warmup=60):
+    """What plain streaming kernels of the vendor's library reach on this box with the merge step's mix of reads and
+    writes, beside which the merge kernel's figure is to be read: HBM efficiency falls with the share of writes
+    (bus turn-arounds), so a kernel that reads 6 bytes and writes 4 per element cannot be priced like one that
+    only reads.  (1) torch's ``acc.add_(blk)`` on the merge step's operands: fp32 read + 16-bit read + fp32 write
+    per element, the same bytes as the merge step less its LSE words, three buffer sets rotated; (2) a 1 GiB copy
+    (half reads, half writes); (3) a read-only pass (``sum`` over the fp32 accumulators)."""
+    import torch
+
+    B, H, S, D = 1, 24, 14882, 128
+    g = torch.Generator(device=dev).manual_seed(1)
+    sets = [(torch.randn(B, H, S, D, generator=g, device=dev), torch.randn(B, H, S, D, generator=g, device=dev).bfloat16())
+            for _ in range(SETS)]
+    out = {}
+    t = _time_calls(lambda i: sets[i % SETS][0].add_(sets[i % SETS][1]), steps, warmup)
+    out["add_fp32_bf16_in_place"] = _hbm("yardstick", "torch add_: fp32 [1,24,14882,128] += bf16, in place (6 B read, 4 B written per element)",
+                                         B * H * S * D * 10, t, SETS)
+    t = _time_calls(lambda i: sets[i % SETS][0].sum(), steps, warmup)
+    out["sum_fp32_read_only"] = _hbm("yardstick", "torch sum over fp32 [1,24,14882,128] (reads only)", B * H * S * D * 4, t, SETS)
+    del sets
+    out["copy_1GiB"] = bench_copy(dev)
+    return out
+
+
 def cpu_baseline(q, k, v):
     """torch's CPU SDPA on the host cores over a bounded sample (about 10-30 s) of the same workload."""
     import torch
@@ -392,7 +417,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     singles = {"merge": bench_merge, "fbcache": bench_fbcache, "taylorseer": bench_taylorseer, "sparse": bench_sparse,
-               "ring": bench_ring, "flux": bench_flux, "wan": bench_wan, "shapes": bench_shapes, "copy": bench_copy}
+               "ring": bench_ring, "flux": bench_flux, "wan": bench_wan, "shapes": bench_shapes, "copy": bench_copy,
+               "yardsticks": bench_yardsticks}
     ap.add_argument("--only", choices=["attn"] + list(singles), default=None,
                     help="profiling aid: run just one kernel's timed loop and print its figures")
     args = ap.parse_args()
@@ -456,6 +482,7 @@ def main():
         extras = {"flux_joint_attention": bench_flux(dev)}
         extras.update(bench_ring(dev))
         extras.update(bench_wan(dev))
+        extras.update(bench_shapes(dev))
         extras["block_sparse"] = bench_sparse(dev)
         extras["merge_lse"] = bench_merge(dev)
         extras["fbcache_residual_diff"] = bench_fbcache(dev)

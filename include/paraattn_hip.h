@@ -61,6 +61,9 @@ PA_API const char* pa_last_error(void);
  *   "stream_even"  PARAATTN_STREAM_EVEN=0|1 that kernel's tail cut into shares that begin at the same keys / into equal ranges, -1 = by size
  *   "sparse_pair"  PARAATTN_SPARSE_PAIR=1   1: pa_attn_fwd_blocksparse with 128-row query blocks puts two adjacent blocks into one
  *                                           256-row workgroup that walks the union of their key ranges (head_dim 128)
+ *   "wave_rows"    PARAATTN_WAVE_ROWS=64    64: the kernel with resident workgroups runs as 4 wavefronts of 64 query rows (one per SIMD,
+ *                                           half the LDS reads per flop) instead of 8 wavefronts of 32: the same results bit for
+ *                                           bit, slower as measured, kept for comparison
  * Returns PA_ERR_INVALID for an unknown name or value.
  */
 PA_API int pa_set_tuning(const char* name, int value);
@@ -233,6 +236,15 @@ PA_API size_t pa_attn_fwd_sweep_workspace_bytes(int B, int H, int Sq, int n_bloc
  */
 PA_API size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int D,
                                    const int64_t k_strides[3], const int64_t v_strides[3]);
+
+/*
+ * The same for one particular call: has_kv_len != 0 if it passes per-batch key counts, is_causal as in the
+ * call.  An is_causal launch never cuts its keys (its workgroups differ in length) and asks only for the few
+ * KB of the score bound; pa_attn_fwd_workspace_bytes() reports the largest of the three plans because it does
+ * not see these arguments.  No counterpart in the reference (aten sizes its own scratch).
+ */
+PA_API size_t pa_attn_fwd_call_workspace_bytes(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3],
+                                        const int64_t v_strides[3], int has_kv_len, int is_causal);
 
 /*
  * Block-sparse attention forward: query block i (of q_block rows, counted from

@@ -28,7 +28,7 @@ PA_MASK_BOOL = 1
 PA_MASK_F32 = 2
 PA_MASK_ACT = 3
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -69,6 +69,7 @@ SIGNATURES = {
          _i, _vp, _sz, _vp],
     ),
     "pa_attn_fwd_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _strides, _strides]),
+    "pa_attn_fwd_call_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _strides, _strides, _i, _i]),
     "pa_attn_fwd_sweep": (
         _i,
         [_vp, _ptrs, _ptrs, _i, _i, _vp, _vp, _i, _i, _i, _i, _i, _strides, _strides, _strides, _strides, _f, _vp, _sz, _vp],
@@ -146,7 +147,7 @@ def check(rc, what):
 
 def set_tuning(name, value):
     """Set one tuning / test knob of the attention launches (pa_set_tuning in the header): "no_pipe", "bm",
-    "no_split", "no_xcd_order", "bound", "stream", "stream_even", "sparse_pair".  The PARAATTN_* environment variables only give the initial values."""
+    "no_split", "no_xcd_order", "bound", "stream", "stream_even", "sparse_pair", "wave_rows".  The PARAATTN_* environment variables only give the initial values."""
     check(load().pa_set_tuning(name.encode(), int(value)), "pa_set_tuning")
 
 

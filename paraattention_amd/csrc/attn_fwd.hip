@@ -59,6 +59,7 @@ constexpr float RESCALE_SLACK = 8.0f;
 constexpr int MAX_KEY_SEGS = 16;
 struct StreamPlan {
   int G, R, Gt, L, n_pieces;
+  int xcd_order;  // 1: workgroup numbers are dealt so that each of 8 XCDs holds a contiguous eighth of them
   int nseg, seg_len, tps;  // key segments, keys and key tiles per segment
   const void* kseg[MAX_KEY_SEGS];
   const void* vseg[MAX_KEY_SEGS];
@@ -136,6 +137,9 @@ struct TileIter {
   int nranges;
   int ri;
   int pos, end;
+  int limit;      // keys there are: a listed range is cut there (a list built for a longer key sequence must not
+                  // lead the walk past the tensors' end; the ranges ascend, so the first one beyond it ends the walk)
+  int flag_mask;  // ~3 where a range's first key carries two flag bits (paired query blocks), else ~0
   int one[2];  // storage for the single dense range
   __device__ __forceinline__ void init_dense(int len) {
     one[0] = 0;
@@ -145,6 +149,8 @@ struct TileIter {
     ri = 0;
     pos = 0;
     end = len;
+    limit = len;
+    flag_mask = ~0;
   }
   __device__ __forceinline__ void init_range(int b, int e) {
     ranges = nullptr;
@@ -152,14 +158,23 @@ struct TileIter {
     ri = 0;
     pos = b;
     end = e;
+    limit = e;
+    flag_mask = ~0;
   }
-  __device__ __forceinline__ void init_list(const int32_t* r, int n) {
+  __device__ __forceinline__ void clip() {
+    if (end > limit) end = limit;
+    if ((pos & flag_mask) >= end) ri = nranges;
+  }
+  __device__ __forceinline__ void init_list(const int32_t* r, int n, int key_limit, bool flagged) {
     ranges = r;
     nranges = n;
     ri = 0;
+    limit = key_limit;
+    flag_mask = flagged ? ~3 : ~0;
     if (n > 0) {
       pos = r[0];
       end = r[1];
+      clip();
     } else {
       pos = end = 0;
     }
@@ -178,6 +193,7 @@ struct TileIter {
       if (ri < nranges) {
         pos = ranges[2 * ri];
         end = ranges[2 * ri + 1];
+        clip();
       }
     }
   }
@@ -214,7 +230,7 @@ __device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int he
     const int hm = p.Hm == 1 ? 0 : head;
     const int sidx = hm * nseg + seg;
     const int cnt = p.runs[sidx];
-    it.init_list(p.runs + (size_t)p.Hm * nseg + (size_t)sidx * p.cap * 2, cnt);
+    it.init_list(p.runs + (size_t)p.Hm * nseg + (size_t)sidx * p.cap * 2, cnt, p.Skv, p.pair != 0);
   } else {
     // causal: a workgroup's work grows with its row index, so the longest ones are started first
     if (p.causal) qt = p.n_qtiles - 1 - qt;
@@ -1792,10 +1808,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
 // first copies, S(0), output drain: 5-10 us against 1.7 us per key tile) is hidden behind the
 // neighbouring pieces' MFMA work.  Dense, not causal, no per-batch key counts.
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool BOUNDED>
-__global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const AttnParams p) {
+template <typename T, bool BOUNDED, int RB = 1>
+__global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
-  constexpr int NW = 8, DC = 8, DB = 4;
+  static_assert(RB == 1 || RB == 2, "a wavefront owns 32 or 64 query rows");
+  constexpr int NW = 8 / RB, DC = 8, DB = 4;
+  constexpr int WROWS = 32 * RB;  // query rows of a wavefront: RB blocks of 32
   constexpr int IPW = 16 / NW;  // copy instructions per wavefront and K (V) tile
   constexpr int RS = 4 * NW;    // tile rows between two of them
   if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
@@ -1803,7 +1821,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                    // [2][64][256 B]
   char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
-  char* const sStage = (char*)smem + 4 * TILE_BYTES;  // [8 wavefronts][32 rows][256 B]: finished outputs on their way out
+  char* const sStage = (char*)smem + 4 * TILE_BYTES;  // [NW wavefronts][WROWS rows][256 B]: finished outputs on their way out
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1814,7 +1832,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   // Workgroups are dealt to the 8 XCDs in turn; with G a multiple of 8 each XCD takes a contiguous eighth of the
   // workgroup numbers, so the pieces its 32 workgroups sweep at one time are neighbours (one or two heads, whose
   // K/V tiles then meet in that XCD's L2), and so are its ranges of the tail.
-  const int wg = (sp.G & 7) == 0 ? (int)(blockIdx.x & 7) * (sp.G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int wg = sp.xcd_order ? (int)(blockIdx.x & 7) * (sp.G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
   constexpr uint32_t OOB = PIPE_OOB;
   // What happens once per piece (a new Q, a new K/V descriptor, a finished piece's output) needs many of the
   // kernel's arguments and little else.  Read through `p` the compiler would load them all once, ahead of the
@@ -1922,15 +1940,18 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
     w.row_end = w.row_begin + 256 < Sq ? w.row_begin + 256 : Sq;
     return w;
   };
-  vec8 qf[DC];  // B operand of the first GEMM: the Q rows of the piece whose scores are computed next
+  vec8 qf[RB][DC];  // B operand of the first GEMM: the Q rows of the piece whose scores are computed next
   auto load_q = [&](int piece) __attribute__((always_inline)) {
     const KArgs kp = kargs();
     const Where w = where(kp, piece);
-    int r = w.row_begin + wave * 32 + l32;
-    r = r < w.row_end ? r : w.row_end - 1;
-    const uint16_t* qp = (const uint16_t*)kp->q + w.batch * kp->qs_b + w.head * kp->qs_h + (int64_t)r * kp->qs_s + 8 * hh;
 #pragma unroll
-    for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(qp + 16 * dc);
+    for (int rb = 0; rb < RB; ++rb) {
+      int r = w.row_begin + wave * WROWS + 32 * rb + l32;
+      r = r < w.row_end ? r : w.row_end - 1;
+      const uint16_t* qp = (const uint16_t*)kp->q + w.batch * kp->qs_b + w.head * kp->qs_h + (int64_t)r * kp->qs_s + 8 * hh;
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) qf[rb][dc] = *(const vec8*)(qp + 16 * dc);
+    }
   };
 
   // ---- global -> LDS copies (as in attn_fwd_d128_pipe_kernel); the descriptor follows the tile's piece and segment
@@ -2010,12 +2031,17 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   };
 
   // ---- accumulators ---------------------------------------------------------------------------
-  floatx16 o[DB];
+  floatx16 o[RB][DB];
+  float m_run[RB], l_run[RB];
 #pragma unroll
-  for (int i = 0; i < DB; ++i)
+  for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-  float m_run = BOUNDED ? 0.f : -INFINITY, l_run = 0.f;
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[rb][i][r] = 0.f;
+    m_run[rb] = BOUNDED ? 0.f : -INFINITY;
+    l_run[rb] = 0.f;
+  }
   const float c = p.scale_log2;
 
   auto mask_tail = [&](floatx16& a0, floatx16& a1, int nvalid) __attribute__((always_inline)) {
@@ -2033,110 +2059,120 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
 
   // ---- output of a finished item ---------------------------------------------------------------
   auto finish_item = [&](const Desc& d) __attribute__((always_inline)) {
-    float l_tot;
-    {
-      auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
-      l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
-    }
-    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    const float lse_nat = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
     const KArgs kp = kargs();
     const Where w = where(kp, d.piece);
-    const int my_row = w.row_begin + wave * 32 + l32;
     float* const acc_out = kp->acc_out;
-    if ((d.flags & FULL) && acc_out == nullptr) {
-      // A whole piece's output.  In the accumulator layout a lane holds 8-byte pieces of its row, 16 bytes apart,
-      // and a store instruction would touch 64 of them in 32 rows; staged through this wavefront's own 8 KB of
-      // LDS (16-byte chunks XOR-swizzled by the row, as the tiles are) the same data leaves as whole 256-byte rows,
-      // four per instruction.  Short pieces (cross-attention) store an output every few key tiles, and every
-      // store has to be through before the next barrier (one counter covers tile copies and stores).
-      char* const st = sStage + wave * 8192;
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          u32x2 x;
-          x[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
-          x[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
-          *(u32x2*)(st + l32 * 256 + 16 * ((4 * db + a) ^ (l32 & 15)) + 8 * hh) = x;
-        }
-      uint16_t* const obase = (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h;
-      const int64_t os_s = kp->os_s;
-      const int row0 = w.row_begin + wave * 32;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int r = 4 * i + (lane >> 4), ch = lane & 15;
-        const u32x4 x = *(const u32x4*)(st + r * 256 + 16 * (ch ^ (r & 15)));
-        if (row0 + r < w.row_end) *(u32x4*)(obase + (int64_t)(row0 + r) * os_s + 8 * ch) = x;
+    for (int rb = 0; rb < RB; ++rb) {
+      float l_tot;
+      {
+        auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run[rb]), __float_as_uint(l_run[rb]), false, false);
+        l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
       }
-      float* const lse_out = kp->lse;
-      if (lse_out != nullptr && hh == 0 && my_row < w.row_end)
-        lse_out[((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row] = lse_nat;
-    } else if (my_row < w.row_end) {
-      if (!(d.flags & FULL)) {  // a share of a piece: normalised fp32 partial + LSE into the workspace
-        const int64_t wrow = (int64_t)(2 * wg + ((d.flags & MID) ? 0 : 1)) * 256 + (my_row - w.row_begin);
-        float* wp = kp->ws_out + wrow * 128;
+      const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+      const float lse_nat = l_tot > 0.f ? (m_run[rb] + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+      const int my_row = w.row_begin + wave * WROWS + 32 * rb + l32;
+      if ((d.flags & FULL) && acc_out == nullptr) {
+        // A whole piece's output.  In the accumulator layout a lane holds 8-byte pieces of its row, 16 bytes apart,
+        // and a store instruction would touch 64 of them in 32 rows; staged through this wavefront's own 8 KB of
+        // LDS (16-byte chunks XOR-swizzled by the row, as the tiles are) the same data leaves as whole 256-byte rows,
+        // four per instruction.  Short pieces (cross-attention) store an output every few key tiles, and every
+        // store has to be through before the next barrier (one counter covers tile copies and stores).
+        char* const st = sStage + wave * (WROWS * 256) + rb * 8192;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
           for (int a = 0; a < 4; ++a) {
-            float4 x = {o[db][4 * a] * inv, o[db][4 * a + 1] * inv, o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv};
-            *(float4*)(wp + 32 * db + 8 * a + 4 * hh) = x;
+            u32x2 x;
+            x[0] = T::pack2(o[rb][db][4 * a] * inv, o[rb][db][4 * a + 1] * inv);
+            x[1] = T::pack2(o[rb][db][4 * a + 2] * inv, o[rb][db][4 * a + 3] * inv);
+            *(u32x2*)(st + l32 * 256 + 16 * ((4 * db + a) ^ (l32 & 15)) + 8 * hh) = x;
           }
-        if (hh == 0) kp->ws_lse[wrow] = lse_nat;
-      } else if (acc_out != nullptr) {  // fold into the running (out, lse) pair
-        const int64_t ridx = ((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row;
-        const int acc_first = kp->acc_first;
-        float* const acc_lse = kp->acc_lse;
-        const float old = acc_first ? -INFINITY : acc_lse[ridx];
-        const float mx2 = fmaxf(old, lse_nat);
-        float w_old = 0.f, w_blk = 0.f, lse_new = -INFINITY;
-        if (mx2 > -INFINITY) {
-          const float e_old = __expf(old - mx2), e_blk = __expf(lse_nat - mx2);
-          const float den = e_old + e_blk;
-          w_old = e_old / den;
-          w_blk = e_blk / den * inv;
-          lse_new = mx2 + __logf(den);
+        uint16_t* const obase = (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h;
+        const int64_t os_s = kp->os_s;
+        const int row0 = w.row_begin + wave * WROWS + 32 * rb;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int r = 4 * i + (lane >> 4), ch = lane & 15;
+          const u32x4 x = *(const u32x4*)(st + r * 256 + 16 * (ch ^ (r & 15)));
+          if (row0 + r < w.row_end) *(u32x4*)(obase + (int64_t)(row0 + r) * os_s + 8 * ch) = x;
         }
-        float* ap = acc_out + ridx * 128;
-        uint16_t* op = kp->out ? (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h + (int64_t)my_row * kp->os_s : nullptr;
+        float* const lse_out = kp->lse;
+        if (lse_out != nullptr && hh == 0 && my_row < w.row_end)
+          lse_out[((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row] = lse_nat;
+      } else if (my_row < w.row_end) {
+        if (!(d.flags & FULL)) {  // a share of a piece: normalised fp32 partial + LSE into the workspace
+          const int64_t wrow = (int64_t)(2 * wg + ((d.flags & MID) ? 0 : 1)) * 256 + (my_row - w.row_begin);
+          float* wp = kp->ws_out + wrow * 128;
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+          for (int db = 0; db < DB; ++db)
 #pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            const int d0 = 32 * db + 8 * a + 4 * hh;
-            float4 r = {0.f, 0.f, 0.f, 0.f};
-            if (!acc_first && w_old > 0.f) r = *(const float4*)(ap + d0);
-            r.x = r.x * w_old + o[db][4 * a] * w_blk;
-            r.y = r.y * w_old + o[db][4 * a + 1] * w_blk;
-            r.z = r.z * w_old + o[db][4 * a + 2] * w_blk;
-            r.w = r.w * w_old + o[db][4 * a + 3] * w_blk;
-            if (op) {
-              u32x2 x;
-              x[0] = T::pack2(r.x, r.y);
-              x[1] = T::pack2(r.z, r.w);
-              *(u32x2*)(op + d0) = x;
-            } else {
-              *(float4*)(ap + d0) = r;
+            for (int a = 0; a < 4; ++a) {
+              float4 x = {o[rb][db][4 * a] * inv, o[rb][db][4 * a + 1] * inv, o[rb][db][4 * a + 2] * inv, o[rb][db][4 * a + 3] * inv};
+              *(float4*)(wp + 32 * db + 8 * a + 4 * hh) = x;
             }
+          if (hh == 0) kp->ws_lse[wrow] = lse_nat;
+        } else if (acc_out != nullptr) {  // fold into the running (out, lse) pair
+          const int64_t ridx = ((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row;
+          const int acc_first = kp->acc_first;
+          float* const acc_lse = kp->acc_lse;
+          const float old = acc_first ? -INFINITY : acc_lse[ridx];
+          const float mx2 = fmaxf(old, lse_nat);
+          float w_old = 0.f, w_blk = 0.f, lse_new = -INFINITY;
+          if (mx2 > -INFINITY) {
+            const float e_old = __expf(old - mx2), e_blk = __expf(lse_nat - mx2);
+            const float den = e_old + e_blk;
+            w_old = e_old / den;
+            w_blk = e_blk / den * inv;
+            lse_new = mx2 + __logf(den);
           }
-        if (hh == 0) acc_lse[ridx] = lse_new;
+          float* ap = acc_out + ridx * 128;
+          uint16_t* op = kp->out ? (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h + (int64_t)my_row * kp->os_s : nullptr;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+              const int d0 = 32 * db + 8 * a + 4 * hh;
+              float4 r = {0.f, 0.f, 0.f, 0.f};
+              if (!acc_first && w_old > 0.f) r = *(const float4*)(ap + d0);
+              r.x = r.x * w_old + o[rb][db][4 * a] * w_blk;
+              r.y = r.y * w_old + o[rb][db][4 * a + 1] * w_blk;
+              r.z = r.z * w_old + o[rb][db][4 * a + 2] * w_blk;
+              r.w = r.w * w_old + o[rb][db][4 * a + 3] * w_blk;
+              if (op) {
+                u32x2 x;
+                x[0] = T::pack2(r.x, r.y);
+                x[1] = T::pack2(r.z, r.w);
+                *(u32x2*)(op + d0) = x;
+              } else {
+                *(float4*)(ap + d0) = r;
+              }
+            }
+          if (hh == 0) acc_lse[ridx] = lse_new;
+        }
       }
     }
     // the next item starts from nothing
 #pragma unroll
-    for (int i = 0; i < DB; ++i)
+    for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-    m_run = BOUNDED ? 0.f : -INFINITY;
-    l_run = 0.f;
+      for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[rb][i][r] = 0.f;
+      m_run[rb] = BOUNDED ? 0.f : -INFINITY;
+      l_run[rb] = 0.f;
+    }
   };
 
   vec8 f[8];          // ring of 8 operand fragments
-  floatx16 sn0, sn1;  // S(j+1) (keys 0..31, 32..63)
-  float mx = 0.f;     // row maximum of S(j), masked, unscaled
+  floatx16 sn[RB][2];  // S(j+1) per row block (keys 0..31, 32..63)
+  float mx[RB];        // row maximum of S(j), masked, unscaled
 #pragma unroll
-  for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+  for (int rb = 0; rb < RB; ++rb) {
+    mx[rb] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sn[rb][0][r] = sn[rb][1][r] = 0.f;
+  }
 
   // ---- prologue: Q of the first piece; K0, V0, K1 copies; S(0) and its row maximum -------------------
   load_q(cur.piece);
@@ -2155,20 +2191,24 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
   for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(sK, 0, dc);
 #pragma unroll
   for (int dc = 0; dc < DC; ++dc) {
-    sn0 = T::mfma32(f[dc], qf[dc], sn0);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) sn[rb][0] = T::mfma32(f[dc], qf[rb][dc], sn[rb][0]);
     f[dc] = read_k(sK, 1, dc);
   }
 #pragma unroll
-  for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
-  {
-    const int nv0 = valid_keys(cur.n0);
-    if (nv0 < BN) mask_tail(sn0, sn1, nv0);
-  }
-  if constexpr (!BOUNDED) {
-    float m2 = fmaxf(sn0[0], sn1[0]);
+  for (int dc = 0; dc < DC; ++dc)
 #pragma unroll
-    for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
-    mx = across(m2);
+    for (int rb = 0; rb < RB; ++rb) sn[rb][1] = T::mfma32(f[dc], qf[rb][dc], sn[rb][1]);
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int nv0 = valid_keys(cur.n0);
+    if (nv0 < BN) mask_tail(sn[rb][0], sn[rb][1], nv0);
+    if constexpr (!BOUNDED) {
+      float m2 = fmaxf(sn[rb][0][0], sn[rb][1][0]);
+#pragma unroll
+      for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn[rb][0][r]), sn[rb][1][r]);
+      mx[rb] = across(m2);
+    }
   }
   // the scores of the second tile already belong to another piece: its Q replaces the first piece's
   if (nxt.piece >= 0 && nxt.piece != cur.piece) load_q(nxt.piece);
@@ -2181,122 +2221,272 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_stream_kernel(const Attn
     constexpr bool inside = decltype(INSIDE)::value;
     const char* tV = sV + par * TILE_BYTES;
     const char* tKn = sK + (par ^ 1) * TILE_BYTES;
-    floatx16 c0 = sn0, c1 = sn1;  // S(j)
+    if constexpr (RB == 1) {
+        floatx16 c0 = sn[0][0], c1 = sn[0][1];  // S(j)
 
-    // everything fetched so far has landed (tile copies, a new piece's Q, a finished piece's stores);
-    // after the barrier nobody still reads what comes next
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
+      // everything fetched so far has landed (tile copies, a new piece's Q, a finished piece's stores);
+      // after the barrier nobody still reads what comes next
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
 
 #pragma unroll
-    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
+      for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
 
-    if constexpr (!BOUNDED) {
-      const float mx_s = mx * c;
-      if (__any(mx_s > m_run + RESCALE_SLACK)) {
-        const float m_new = fmaxf(m_run, mx_s);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        l_run *= alpha;
+      if constexpr (!BOUNDED) {
+        const float mx_s = mx[0] * c;
+        if (__any(mx_s > m_run[0] + RESCALE_SLACK)) {
+          const float m_new = fmaxf(m_run[0], mx_s);
+          const float alpha = __builtin_amdgcn_exp2f(m_run[0] - m_new);
+          l_run[0] *= alpha;
 #pragma unroll
-        for (int i = 0; i < DB; ++i)
+          for (int i = 0; i < DB; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
-        m_run = m_new;
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- stage A: S(j+1) = K(j+1) Q^T, the copies of K(j+2) and V(j+1), the softmax of S(j) -------
-    uint32_t pk0[8], pk1[8];
-    float lsum = 0.f;
-    float tf[2][2], te[2][2];
-    auto expo_slot = [&](int n) __attribute__((always_inline)) {
-      if (n >= 2 && n < 18) {
-        const int j = n - 2;
-        lsum += te[j & 1][0] + te[j & 1][1];
-        asm volatile("" : "+v"(lsum));  // the addition stays in its slot (left alone it sinks behind the last MFMA: -1.6 %)
-        (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
-      }
-      if (n >= 1 && n < 17) {
-        const int j = n - 1;
-        te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
-        te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
-      }
-      if (n < 16) {
-        const floatx16& cs = n < 8 ? c0 : c1;
-        tf[n & 1][0] = __builtin_fmaf(cs[2 * (n & 7)], c, -m_run);
-        tf[n & 1][1] = __builtin_fmaf(cs[2 * (n & 7) + 1], c, -m_run);
-      }
-    };
-#pragma unroll
-    for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
-#pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
-      else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
-      if (g < IPW) dma_k1(par, nx2.n0, g, inside);
-      else if (g < 2 * IPW) dma_v1(par ^ 1, nxt.n0, g - IPW, inside);
-      f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      if (g & 1) sn1 = T::mfma32(f[g], qf[4 + (g >> 1)], sn1);
-      else sn0 = T::mfma32(f[g], qf[4 + (g >> 1)], sn0);
-      f[g] = read_vt(tV, 0, g >> 2, g & 3);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if constexpr (!inside) {
-      const int nv1 = valid_keys(nxt.n0);
-      if (nv1 < BN) mask_tail(sn0, sn1, nv1);  // ragged or absent tile j+1
-      // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
-      if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // The softmax of S(j) begins here, not under the MFMAs of stage A: VALU work between the MFMAs of the first
-    // GEMM costs more than it hides (measured: -3.5 %): the first six slots, which the first PV MFMA needs, in front
-    // of it, then one slot under each of the next twelve PV MFMAs.
-#pragma unroll
-    for (int n = 0; n < 6; ++n) expo_slot(n);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- stage B: O^T += V(j)^T P(j)^T, the rest of the softmax, the row maximum of S(j+1) ----------
-    float mxa = fmaxf(sn0[0], sn0[1]), mxb = fmaxf(sn1[0], sn1[1]);
-#pragma unroll
-    for (int cc = 0; cc < 2; ++cc) {
-      u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
-      vec8 bfrag = __builtin_bit_cast(vec8, bw);
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int g = cc * 4 + db;
-        o[db] = T::mfma32(f[g], bfrag, o[db]);
-        f[g] = read_vt(tV, 1, cc, db);
-        expo_slot(6 + g);
-        if constexpr (!BOUNDED) {
-          if (g < 4) {
-          } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
-          else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
+            for (int r = 0; r < 16; ++r) o[0][i][r] *= alpha;
+          m_run[0] = m_new;
         }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- stage A: S(j+1) = K(j+1) Q^T, the copies of K(j+2) and V(j+1), the softmax of S(j) -------
+      uint32_t pk0[8], pk1[8];
+      float lsum = 0.f;
+      float tf[2][2], te[2][2];
+      auto expo_slot = [&](int n) __attribute__((always_inline)) {
+        if (n >= 2 && n < 18) {
+          const int j = n - 2;
+          lsum += te[j & 1][0] + te[j & 1][1];
+          asm volatile("" : "+v"(lsum));  // the addition stays in its slot (left alone it sinks behind the last MFMA: -1.6 %)
+          (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
+        }
+        if (n >= 1 && n < 17) {
+          const int j = n - 1;
+          te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
+          te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
+        }
+        if (n < 16) {
+          const floatx16& cs = n < 8 ? c0 : c1;
+          tf[n & 1][0] = __builtin_fmaf(cs[2 * (n & 7)], c, -m_run[0]);
+          tf[n & 1][1] = __builtin_fmaf(cs[2 * (n & 7) + 1], c, -m_run[0]);
+        }
+      };
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sn[0][0][r] = sn[0][1][r] = 0.f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        if (g & 1) sn[0][1] = T::mfma32(f[g], qf[0][g >> 1], sn[0][1]);
+        else sn[0][0] = T::mfma32(f[g], qf[0][g >> 1], sn[0][0]);
+        if (g < IPW) dma_k1(par, nx2.n0, g, inside);
+        else if (g < 2 * IPW) dma_v1(par ^ 1, nxt.n0, g - IPW, inside);
+        f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
         __builtin_amdgcn_sched_barrier(0);
       }
-    }
 #pragma unroll
-    for (int cc = 0; cc < 2; ++cc) {
-      u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
-      vec8 bfrag = __builtin_bit_cast(vec8, bw);
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int g = cc * 4 + db;
-        o[db] = T::mfma32(f[g], bfrag, o[db]);
-        if (g < 4) expo_slot(14 + g);
-        if constexpr (!BOUNDED) {
-          if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
-        }
+      for (int g = 0; g < 8; ++g) {
+        if (g & 1) sn[0][1] = T::mfma32(f[g], qf[0][4 + (g >> 1)], sn[0][1]);
+        else sn[0][0] = T::mfma32(f[g], qf[0][4 + (g >> 1)], sn[0][0]);
+        f[g] = read_vt(tV, 0, g >> 2, g & 3);
         __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (!inside) {
+        const int nv1 = valid_keys(nxt.n0);
+        if (nv1 < BN) mask_tail(sn[0][0], sn[0][1], nv1);  // ragged or absent tile j+1
+        // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
+        if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // The softmax of S(j) begins here, not under the MFMAs of stage A: VALU work between the MFMAs of the first
+      // GEMM costs more than it hides (measured: -3.5 %): the first six slots, which the first PV MFMA needs, in front
+      // of it, then one slot under each of the next twelve PV MFMAs.
+#pragma unroll
+      for (int n = 0; n < 6; ++n) expo_slot(n);
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- stage B: O^T += V(j)^T P(j)^T, the rest of the softmax, the row maximum of S(j+1) ----------
+      float mxa = fmaxf(sn[0][0][0], sn[0][0][1]), mxb = fmaxf(sn[0][1][0], sn[0][1][1]);
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
+        vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const int g = cc * 4 + db;
+          o[0][db] = T::mfma32(f[g], bfrag, o[0][db]);
+          f[g] = read_vt(tV, 1, cc, db);
+          expo_slot(6 + g);
+          if constexpr (!BOUNDED) {
+            if (g < 4) {
+            } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn[0][0][4 * g - 14]), sn[0][0][4 * g - 13]), sn[0][0][4 * g - 12]), sn[0][0][4 * g - 11]);
+            else mxa = fmaxf(fmaxf(mxa, sn[0][0][14]), sn[0][0][15]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
+        vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const int g = cc * 4 + db;
+          o[0][db] = T::mfma32(f[g], bfrag, o[0][db]);
+          if (g < 4) expo_slot(14 + g);
+          if constexpr (!BOUNDED) {
+            if (g > 0) mxb = fmaxf(fmaxf(mxb, sn[0][1][2 * g]), sn[0][1][2 * g + 1]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      l_run[0] += lsum;
+      if constexpr (!BOUNDED) mx[0] = across(fmaxf(mxa, mxb));
+
+    } else {
+      // ---- 64 query rows per wavefront, one wavefront per SIMD ------------------------------------------
+      // Every K and V^T fragment read from LDS feeds two MFMAs (one per row block), so the workgroup reads half
+      // the LDS bytes per flop of the 32-row form.  No second wavefront shares the SIMD: the softmax of S(j) has
+      // to run under this wavefront's own MFMAs, spread evenly over both GEMMs (34 slots under MFMAs 0..59 of
+      // the iteration's 64), each group of 16 probabilities finished just before the PV MFMAs that take it.
+      floatx16 cs[RB][2];  // S(j)
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        cs[rb][0] = sn[rb][0];
+        cs[rb][1] = sn[rb][1];
+      }
+
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
+
+      if constexpr (!BOUNDED) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const float mx_s = mx[rb] * c;
+          if (__any(mx_s > m_run[rb] + RESCALE_SLACK)) {
+            const float m_new = fmaxf(m_run[rb], mx_s);
+            const float alpha = __builtin_amdgcn_exp2f(m_run[rb] - m_new);
+            l_run[rb] *= alpha;
+#pragma unroll
+            for (int i = 0; i < DB; ++i)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) o[rb][i][r] *= alpha;
+            m_run[rb] = m_new;
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+
+      // Softmax of S(j) in 32 pairs of scores, in the order the second GEMM takes them: pair n belongs to the
+      // 16-key chunk n / 8 (key half t = n / 16, chunk cc of it), row block (n / 4) % 2, registers 8 cc + 2 (n % 4).
+      // A pair passes three slots: scale, exponentials, sum + pack.
+      uint32_t pk[RB][2][8];
+      float lsum[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) lsum[rb] = 0.f;
+      float tf[2][2], te[2][2];
+      auto expo_slot = [&](int n) __attribute__((always_inline)) {
+        if (n >= 2 && n < 34) {
+          const int j = n - 2, rb = (j >> 2) & 1, k = j >> 3;
+          lsum[rb] += te[j & 1][0] + te[j & 1][1];
+          asm volatile("" : "+v"(lsum[rb]));
+          pk[rb][k >> 1][4 * (k & 1) + (j & 3)] = T::pack2(te[j & 1][0], te[j & 1][1]);
+        }
+        if (n >= 1 && n < 33) {
+          const int j = n - 1;
+          te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
+          te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
+        }
+        if (n < 32) {
+          const int rb = (n >> 2) & 1, k = n >> 3;
+          const floatx16& src = cs[rb][k >> 1];
+          const int r0 = 8 * (k & 1) + 2 * (n & 3);
+          tf[n & 1][0] = __builtin_fmaf(src[r0], c, -m_run[rb]);
+          tf[n & 1][1] = __builtin_fmaf(src[r0 + 1], c, -m_run[rb]);
+        }
+      };
+      // slots finished once MFMA q of the iteration has been issued
+      auto slots_done = [](int q) constexpr { return q < 0 ? 0 : ((q + 1) * 34 / 60 < 34 ? (q + 1) * 34 / 60 : 34); };
+      auto run_slots = [&](int q) __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = slots_done(q - 1); n < slots_done(q); ++n) expo_slot(n);
+      };
+
+      // ---- S(j+1) = K(j+1) Q^T: 32 MFMAs; the copies of K(j+2) and V(j+1) behind the first eight -------
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sn[rb][0][r] = sn[rb][1][r] = 0.f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const int q = 2 * g + rb;
+          sn[rb][g & 1] = T::mfma32(f[g], qf[rb][g >> 1], sn[rb][g & 1]);
+          if (q < IPW) dma_k1(par, nx2.n0, q, inside);
+          else if (q < 2 * IPW) dma_v1(par ^ 1, nxt.n0, q - IPW, inside);
+          if (rb == RB - 1) f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
+          run_slots(q);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const int q = 16 + 2 * g + rb;
+          sn[rb][g & 1] = T::mfma32(f[g], qf[rb][4 + (g >> 1)], sn[rb][g & 1]);
+          if (rb == RB - 1) f[g] = read_vt(tV, 0, g >> 2, g & 3);
+          run_slots(q);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if constexpr (!inside) {
+        const int nv1 = valid_keys(nxt.n0);
+        if (nv1 < BN) {  // ragged or absent tile j+1
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) mask_tail(sn[rb][0], sn[rb][1], nv1);
+        }
+        // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
+        if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- O^T += V(j)^T P(j)^T: 32 MFMAs, chunk by chunk of 16 keys, row block 0 then 1 with the same fragments;
+      // the rest of the softmax, and the row maxima of S(j+1) ----------------------------------------
+      float mxv[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) mxv[rb] = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            u32x4 bw = {pk[rb][t][4 * cc], pk[rb][t][4 * cc + 1], pk[rb][t][4 * cc + 2], pk[rb][t][4 * cc + 3]};
+            vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+              const int u = 8 * (2 * t + cc) + 4 * rb + db;  // MFMA 32 + u of the iteration
+              const int g = cc * 4 + db;
+              o[rb][db] = T::mfma32(f[g], bfrag, o[rb][db]);
+              if (t == 0 && rb == RB - 1) f[g] = read_vt(tV, 1, cc, db);
+              run_slots(32 + u);
+              if constexpr (!BOUNDED) {
+                const floatx16& sx = sn[u >> 4][(u >> 3) & 1];
+                const int i = u & 7;
+                mxv[u >> 4] = fmaxf(fmaxf(mxv[u >> 4], sx[2 * i]), sx[2 * i + 1]);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        l_run[rb] += lsum[rb];
+        if constexpr (!BOUNDED) mx[rb] = across(mxv[rb]);
+      }
     }
-    l_run += lsum;
-    if constexpr (!BOUNDED) mx = across(fmaxf(mxa, mxb));
 
     if constexpr (inside) {
       cur.n0 = nxt.n0;
@@ -2893,6 +3083,10 @@ struct SplitPlan {
   int tiles, s;
   double rounds;
 };
+// The planners' measured constants (microseconds per key tile, what 256-row workgroups gain over 128-row ones, the
+// dealing of workgroups to 8 XCDs) are MI355X's: 256 compute units in 8 XCDs.  On a device that reports another
+// compute-unit count the launches fall back to plain plans: no key split priced by those constants, no XCD order.
+static bool mi355x_layout() { return device_cus() == 256; }
 static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bool allow) {
   if (slots <= 0) return {0, 1, 1.0};  // no device to ask: no estimate, no split
   SplitPlan best = {0, 1, (double)((n_tiles + slots - 1) / slots)};
@@ -2926,8 +3120,9 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
 //   PARAATTN_STREAM=0|1      "stream"        never / wherever possible the resident-workgroup kernel (-1 = by shape)
 //   PARAATTN_STREAM_EVEN=0|1 "stream_even"   its tail cut into shares that begin at the same keys / into equal ranges (-1 = by size)
 //   PARAATTN_SPARSE_PAIR=1   "sparse_pair"   block-sparse with 128-row query blocks: two adjacent blocks per 256-row workgroup
+//   PARAATTN_WAVE_ROWS=64    "wave_rows"     the resident-workgroup kernel as 4 wavefronts of 64 query rows instead of 8 of 32
 struct Tuning {
-  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair;
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair, wave_rows;
 };
 static Tuning& tuning() {
   static Tuning t;
@@ -2947,6 +3142,7 @@ static Tuning& tuning() {
     const int se = num("PARAATTN_STREAM_EVEN", -1);
     t.stream_even = se == 0 || se == 1 ? se : -1;
     t.sparse_pair = num("PARAATTN_SPARSE_PAIR", 0) == 1;
+    t.wave_rows = num("PARAATTN_WAVE_ROWS", 0) == 64 ? 64 : 0;
     return true;
   }();
   (void)init;
@@ -2966,6 +3162,7 @@ extern "C" int pa_set_tuning(const char* name, int value) {
   else if (!strcmp(name, "stream")) t.stream = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "stream_even")) t.stream_even = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "sparse_pair")) t.sparse_pair = value == 1;
+  else if (!strcmp(name, "wave_rows")) t.wave_rows = value == 64 ? 64 : 0;
   else PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: unknown knob '%s'", name);
   return PA_OK;
 }
@@ -3005,7 +3202,7 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
   }
   const int cus = device_cus();
   // (causal workgroups differ in length: the rounds estimate does not apply, no split)
-  const bool allow = cus > 0 && !p.causal && !tuning().no_split && (ws_needed != nullptr || ws_bytes > 0);
+  const bool allow = cus > 0 && mi355x_layout() && !p.causal && !tuning().no_split && (ws_needed != nullptr || ws_bytes > 0);
   const int kv_tiles = (p.Skv + BN - 1) / BN;
   const int64_t bh = (int64_t)p.B * p.H;
   const int64_t n128 = bh * ((p.Sq + 127) / 128), n256 = bh * ((p.Sq + 255) / 256);
@@ -3020,7 +3217,7 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
   if (cus > 0 && p128.s == 1 && n128 % (2 * cus) != 0 && n128 % (2 * cus) <= cus) r128 -= 0.33;
   // measured throughput of a full round of 256-row workgroups against one of 128-row workgroups:
   // +4..10 % from 4608 keys up, -4 % at 512 keys
-  const double gain256 = kv_tiles >= 32 ? 1.055 : 0.95;
+  const double gain256 = !mi355x_layout() ? 1.0 : kv_tiles >= 32 ? 1.055 : 0.95;
   bool use256 = cus > 0 && n256 >= cus && r256 / gain256 < r128;
   if (forced == 128) use256 = false;
   if (forced == 256) use256 = true;
@@ -3090,6 +3287,7 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   // and resident workgroups hide what a workgroup per piece pays per piece and cut a ragged last round finely.
   StreamPlan& st = p.st;
   st.G = cus;
+  st.xcd_order = mi355x_layout() && (cus & 7) == 0;
   st.R = P / st.G;
   st.L = L;
   st.n_pieces = P;
@@ -3142,26 +3340,33 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   return true;
 }
 
-template <typename T>
-static int launch_stream(const AttnParams& p, hipStream_t stream) {
-  if (p.out == nullptr && p.acc_out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
+template <typename T, int RB>
+static int launch_stream_rb(const AttnParams& p, hipStream_t stream) {
   const size_t smem = 4 * TILE_BYTES + 8 * 8192;  // two K and two V tiles, and a staging area for outputs
   static bool attr_done[PA_MAX_DEVICES][2] = {};  // benign race: the call is idempotent
   const int dev = current_device();
   for (int b = 0; b < 2; ++b) {
     if (b == 1 && p.bound_flag == nullptr) break;
     if (dev >= 0 && attr_done[dev][b]) continue;
-    const void* fn = b ? (const void*)attn_fwd_d128_stream_kernel<T, true> : (const void*)attn_fwd_d128_stream_kernel<T, false>;
+    const void* fn = b ? (const void*)attn_fwd_d128_stream_kernel<T, true, RB> : (const void*)attn_fwd_d128_stream_kernel<T, false, RB>;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     if (dev >= 0) attr_done[dev][b] = true;
   }
   if (p.bound_flag != nullptr) {  // one of the two variants leaves at once
-    hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, true>), dim3((unsigned)p.st.G), dim3(512), smem, stream, p);
+    hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, true, RB>), dim3((unsigned)p.st.G), dim3(512 / RB), smem, stream, p);
     PA_CHECK_LAUNCH("attention kernel (resident workgroups, bounded scores)");
   }
-  hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, false>), dim3((unsigned)p.st.G), dim3(512), smem, stream, p);
+  hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, false, RB>), dim3((unsigned)p.st.G), dim3(512 / RB), smem, stream, p);
   PA_CHECK_LAUNCH("attention kernel (resident workgroups)");
+  return PA_OK;
+}
+
+template <typename T>
+static int launch_stream(const AttnParams& p, hipStream_t stream) {
+  if (p.out == nullptr && p.acc_out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
+  const int rc = tuning().wave_rows == 64 ? launch_stream_rb<T, 2>(p, stream) : launch_stream_rb<T, 1>(p, stream);
+  if (rc != PA_OK) return rc;
   const int p_tail = p.st.n_pieces - p.st.R * p.st.G;
   if (p_tail > 0 && p.st.Gt != p_tail) {
     hipLaunchKernelGGL((attn_stream_merge_kernel<T>), dim3((unsigned)p_tail * 16), dim3(256), 0, stream, p);
@@ -3341,16 +3546,19 @@ extern "C" size_t pa_attn_fwd_sweep_workspace_bytes(int B, int H, int Sq, int n_
 
 // Workspace of a dense call: partial results of the plan plus the score bound's words.  which = 0: the plan of a
 // call without per-batch key counts and is_causal (resident workgroups where they apply); 1: the plan of a call
-// with either; 2: the larger.
+// with per-batch key counts (one workgroup per query tile, key-split tail); 2: the plan of an is_causal call
+// (never split: only the score bound's words); WS_ANY: the largest of them.
+constexpr int WS_ANY = 3;
 static size_t dense_ws_need(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3], const int64_t v_strides[3], int which) {
   const int64_t zero[3] = {0, 0, 0};
   size_t best = 0;
-  for (int plan = 0; plan < 2; ++plan) {
-    if (which != 2 && which != plan) continue;
+  for (int plan = 0; plan < 3; ++plan) {
+    if (which != WS_ANY && which != plan) continue;
     AttnParams p;
     fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
+    p.causal = plan == 2;
     size_t need = 0;
-    if (plan == 1 || !plan_stream(p, D, nullptr, 0, true, &need)) {
+    if (plan != 0 || !plan_stream(p, D, nullptr, 0, true, &need)) {
       need = 0;
       choose_kernel(p, D, 256, true, 0, &need);
     }
@@ -3365,7 +3573,13 @@ extern "C" size_t pa_attn_fwd_workspace_bytes(int B, int H, int Sq, int Skv, int
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || (D != 128 && D != 64) || !k_strides || !v_strides) return 0;
   // the larger of what the two plans ask for: which of them a call gets depends on arguments this function does not
   // see (per-batch key counts and is_causal go to attn_fwd_d128_pipe_kernel)
-  return dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, 2);
+  return dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, WS_ANY);
+}
+
+extern "C" size_t pa_attn_fwd_call_workspace_bytes(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3],
+                                                   const int64_t v_strides[3], int has_kv_len, int is_causal) {
+  if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || (D != 128 && D != 64) || !k_strides || !v_strides) return 0;
+  return dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, is_causal ? 2 : has_kv_len ? 1 : 0);
 }
 
 // The generic kernel with an attention mask (any head_dim it is built for, any strides).
@@ -3485,7 +3699,7 @@ extern "C" int pa_attn_fwd_lse_noalloc(const void* q, const void* k, const void*
                                        float scale, const int32_t* kv_len, int is_causal, void* stream) {
   // what the same problem would ask of a caller's workspace (0 for sizes that use none)
   const bool shaped = B > 0 && H > 0 && Sq > 0 && Skv > 0 && (D == 128 || D == 64) && k_strides && v_strides;
-  const size_t need = shaped ? dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, kv_len != nullptr || is_causal ? 1 : 0) : 0;
+  const size_t need = shaped ? dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, is_causal ? 2 : kv_len != nullptr ? 1 : 0) : 0;
   if (need > (size_t)PA_NOALLOC_SCRATCH_BYTES)
     PA_FAIL(PA_ERR_WORKSPACE, "this problem's launch plan needs %zu bytes of scratch, the static buffer holds %zu: "
             "call pa_attn_fwd_lse_ws with a workspace of your own", need, (size_t)PA_NOALLOC_SCRATCH_BYTES);
@@ -3561,7 +3775,7 @@ static int blocksparse_launch(const void* q, const void* k, const void* v, void*
   const int q_hi = q_lo + nQ * q_block;
   const int tiles_right = (Sq - q_hi + p.bm - 1) / p.bm;
   p.n_qtiles = p.tiles_left + nQ * p.tiles_per_block + tiles_right;
-  if (D == 128 && p.pipe && !tuning().no_xcd_order)
+  if (D == 128 && p.pipe && !tuning().no_xcd_order && mi355x_layout())
     p.xcd_chunk = (int)(((int64_t)B * H * p.n_qtiles + 7) / 8);
   return dispatch_attn<true>(p, dtype, D, (hipStream_t)stream);
 }

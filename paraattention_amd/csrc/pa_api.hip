@@ -8,6 +8,6 @@ char* error_slot() {
 }
 }  // namespace pa
 
-extern "C" int pa_abi_version(void) { return 3; }
+extern "C" int pa_abi_version(void) { return 4; }
 
 extern "C" const char* pa_last_error(void) { return pa::error_slot(); }

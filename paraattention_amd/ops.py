@@ -113,9 +113,7 @@ def _dense_forward(query, key, value, scale, want_lse, kv_len=None, is_causal=Fa
         # scratch for the score bound and the key-split tail of the launch (torch's caching allocator:
         # no hipMalloc in the steady state); its lifetime on the launch stream is the allocator's business
         ks, vs = _lib.strides3(k), _lib.strides3(v)
-        ws_bytes = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, ks, vs)
-        if is_causal:  # causal launches never split: the score bound's few KB at the front are all they use
-            ws_bytes = min(ws_bytes, 16384)
+        ws_bytes = lib.pa_attn_fwd_call_workspace_bytes(B, H, Sq, Skv, D, ks, vs, 0 if kv_len is None else 1, 1 if is_causal else 0)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
         rc = lib.pa_attn_fwd_lse_ws(
             _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _DTYPE_CODE[q.dtype], B, H, Sq, Skv, D,

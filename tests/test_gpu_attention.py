@@ -390,7 +390,8 @@ def test_key_split_tail(cuda, bm, tuning):
 
 @pytest.mark.parametrize("even", [-1, 0, 1])
 @pytest.mark.parametrize("bound", [0, 1])
-def test_resident_workgroup_kernel(cuda, even, bound, tuning):
+@pytest.mark.parametrize("wave_rows", [32, 64])
+def test_resident_workgroup_kernel(cuda, even, bound, wave_rows, tuning):
     """The kernel whose workgroups stay resident and walk a list of pieces as one stream of key tiles, forced on
     for every shape here: fewer pieces than compute units (every piece cut into ranges), a few pieces more than a
     whole number of rounds (whole pieces, then a tail cut evenly or into shares that begin at the same keys),
@@ -400,6 +401,7 @@ def test_resident_workgroup_kernel(cuda, even, bound, tuning):
     tuning("stream", 1)
     tuning("stream_even", even)
     tuning("bound", bound)
+    tuning("wave_rows", wave_rows)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     op = torch.ops.para_attn.attention_forward_with_lse
     shapes = [(1, 2, 300, 434), (2, 3, 129, 1000), (1, 1, 64, 64), (1, 3, 1000, 77), (2, 2, 700, 128), (1, 5, 2000, 40),
@@ -489,6 +491,46 @@ def test_score_bound_variants(cuda, dtype, D, bm, tuning):
         tuning("bound", 0)
         out0, lse0 = op(q.to(cuda), k.to(cuda), v.to(cuda))
         assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
+
+
+@pytest.mark.parametrize("D,bm", [(128, "256"), (64, "128"), (64, "256")])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("side", ["under", "over"])
+def test_score_bound_at_the_limit(cuda, dtype, D, bm, side, tuning):
+    """The score bound where dropping the running maximum is riskiest: every q and k row has the same norm, chosen so
+    that the device-computed bound |q| |k| scale log2(e) lands just under the limit (about 58 of 60 for bf16, 13.5 of
+    14 for fp16: the variant without a maximum runs) or just over it (the variant with the maximum runs), and some
+    query rows meet one key aligned with them and one opposed to them, so a single row realises scores at both
+    ends of the bound (exp2 of +58 and of -58 in one sum).  Against the fp64 oracle and against the launch with the
+    bound switched off."""
+    tuning("bm", int(bm))
+    limit = 60.0 if dtype == torch.bfloat16 else 14.0
+    target = limit - (2.0 if dtype == torch.bfloat16 else 0.5) if side == "under" else limit + (2.0 if dtype == torch.bfloat16 else 0.5)
+    c = D ** -0.5 * 1.4426950408889634
+    norm = (target / c) ** 0.5
+    B, H, Sq, Skv = 1, 2, 600, 1300
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=77, dtype=torch.float32)
+    q = q / q.norm(dim=-1, keepdim=True) * norm
+    k = k / k.norm(dim=-1, keepdim=True) * norm
+    planted = [0, 31, 32, 255, 256, 300, 599]  # first and last rows of wavefronts and workgroups among them
+    for n, i in enumerate(planted):
+        k[:, :, 7 + 64 * n] = q[:, :, i]         # aligned: the row's largest score, +bound
+        k[:, :, 1299 - 97 * n] = -q[:, :, i]     # opposed: its smallest, -bound
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    # what the device computes from the rounded operands (largest row norms, fp32)
+    bound = q.float().norm(dim=-1).max().item() * k.float().norm(dim=-1).max().item() * c
+    assert (limit - 3 < bound < limit - 0.2) if side == "under" else (limit + 0.2 < bound < limit + 3), bound
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    s = np.einsum("bhid,bhjd->bhij", q.float().numpy().astype(np.float64), k.float().numpy().astype(np.float64)) * c
+    assert s[:, :, planted].max() > bound - 0.5 and s[:, :, planted].min() < -bound + 0.5  # both ends are realised
+    op = torch.ops.para_attn.attention_forward_with_lse
+    tuning("bound", 1)
+    out, lse = op(q.to(cuda), k.to(cuda), v.to(cuda))
+    _check(out, lse, ref_out, ref_lse, f"bound {bound:.2f} of {limit} ({side}) {dtype} D={D}")
+    tuning("bound", 0)
+    out0, lse0 = op(q.to(cuda), k.to(cuda), v.to(cuda))
+    _check(out0, lse0, ref_out, ref_lse, f"no bound, {bound:.2f} {dtype} D={D}")
+    assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-3
 
 
 CAUSAL = [(1, 2, 1, 1), (1, 1, 17, 17), (2, 2, 64, 64), (1, 2, 129, 129), (1, 1, 300, 300), (1, 2, 700, 700),

@@ -132,6 +132,11 @@ def test_prebuilt_runs_entry(cuda):
             assert torch.equal(out, w_out) and torch.equal(lse, w_lse)
         with pytest.raises(ValueError):
             torch.ops.para_attn.attention_forward_block_sparse_runs(q, k, v, runs[:10], hm, 4, 6, *q_range)
+        # ranges built for a longer key sequence (a longer dense right margin) are cut at the keys there are:
+        # the walk never leaves the tensors, and here the cut lists are those of the true length
+        longer = torch.ops.para_attn.block_sparse_key_runs(bm.to(cuda), Skv + 200, *kv_range)
+        out, lse = torch.ops.para_attn.attention_forward_block_sparse_runs(q, k, v, longer, hm, 4, 6, *q_range)
+        assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
     bm = torch.rand((4, 6), generator=g) < 0.5
     bm[:, 0] = True
     with paraattention_amd.StructSparseAttnMode(sparse_mask=bm, sparse_range_query=q_range, sparse_range_key_value=kv_range) as mode:
@@ -147,6 +152,15 @@ def test_prebuilt_runs_entry(cuda):
         o3 = torch.nn.functional.scaled_dot_product_attention(q, k, v)
         want3, _ = torch.ops.para_attn.attention_forward_block_sparse(q, k, v, bm.to(cuda), *q_range, *kv_range)
         assert torch.equal(o3, want3) and len(cache) == 1 and next(iter(cache.values())) is not held
+        # a second key length through the same mode: its own entry, and the first one is still there afterwards
+        k2, v2 = k[:, :, : kv_range[1]].contiguous(), v[:, :, : kv_range[1]].contiguous()
+        o4 = torch.nn.functional.scaled_dot_product_attention(q, k2, v2)
+        want4, _ = torch.ops.para_attn.attention_forward_block_sparse(q, k2, v2, bm.to(cuda), *q_range, *kv_range)
+        assert torch.equal(o4, want4) and len(cache) == 2
+        entries = list(cache.values())
+        assert torch.equal(torch.nn.functional.scaled_dot_product_attention(q, k, v), want3)
+        assert torch.equal(torch.nn.functional.scaled_dot_product_attention(q, k2, v2), want4)
+        assert len(cache) == 2 and all(a is b for a, b in zip(cache.values(), entries))  # both served from the cache
 
 
 def test_paired_query_blocks(cuda, tuning):

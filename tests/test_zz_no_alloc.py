@@ -105,3 +105,17 @@ def test_noalloc_refuses_what_the_buffer_cannot_hold(cuda, tuning):
     # the entry with a caller's workspace takes the same problem
     out, lse, _ = _call_ws(lib, q, k, v)
     assert torch.isfinite(lse).all()
+    # with is_causal the same shape is taken: a causal launch never cuts its keys and uses the score bound's few KB only
+    tuning("bound", 1)
+    assert lib.pa_attn_fwd_call_workspace_bytes(B, H, Sq, Skv, D, _lib.strides3(k), _lib.strides3(v), 0, 1) <= 16384
+    assert lib.pa_attn_fwd_call_workspace_bytes(B, H, Sq, Skv, D, _lib.strides3(k), _lib.strides3(v), 1, 0) >= need  # the key-split plan (+ the bound's words)
+    rc, cout, clse = _call_noalloc(lib, q, k, v, causal=1)
+    assert rc == 0, lib.pa_last_error()
+    torch.cuda.synchronize()
+    want_out, want_lse, _ = _call_ws(lib, q, k, v, causal=1)
+    assert torch.equal(cout, want_out) and torch.equal(clse, want_lse)
+    rows = torch.tensor([0, 1, 255, 256, 4097, Skv - 1, Skv, Sq - 1])
+    keep = (torch.arange(Skv)[None, :] <= rows[:, None])[None, None]
+    ref_out, ref_lse = oattn.sdpa_lse_torch_cpu(q[:, :, rows].cpu(), k.cpu(), v.cpu(), attn_mask=keep)
+    assert (cout[:, :, rows.to(cuda)].float().cpu() - ref_out.float()).abs().max().item() <= 2e-2 + 2e-2 * ref_out.float().abs().max().item()
+    assert (clse[:, :, rows.to(cuda)].cpu() - ref_lse).abs().max().item() <= 1e-3
