@@ -36,8 +36,8 @@ def kernel_takes(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=Fal
         return False
     if is_causal and attn_mask is not None:
         return False
-    if query.shape[-1] not in (64, 128) or value.shape[-1] != query.shape[-1]:
-        return False
+    if not (1 <= query.shape[-1] <= 128 and 1 <= value.shape[-1] <= 128) or key.shape[-1] != query.shape[-1]:
+        return False  # 64 and 128 natively, other head_dims up to 128 zero-padded (ops._pad_head_dims)
     if query.requires_grad or key.requires_grad or value.requires_grad:
         return False  # forward only, like the reference's ops (src/para_attn/ops/__init__.py:203-211)
     if attn_mask is not None:

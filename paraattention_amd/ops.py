@@ -53,11 +53,33 @@ def _kernel_ready(t):
     return t
 
 
-def _out_like(query):
+def _native_head_dims(query, value):
+    """The kernels are built for head_dim 64 and 128 with values as wide as the keys; anything else up to 128 runs
+    through them zero-padded (``_pad_head_dims``)."""
+    return query.shape[-1] == value.shape[-1] and query.shape[-1] in (64, 128)
+
+
+def _pad_head_dims(query, key, value, scale):
+    """q, k, v with head_dim zero-padded to 64 or 128 and the scale of the true head_dim.  Zero columns add nothing
+    to q.k, and the padded columns of v give output columns that are dropped, so the result is that of the unpadded
+    problem: head_dim 32, 40, 72, 80, 96 ... and values narrower or wider than the keys (which aten's kernels behind
+    src/para_attn/ops/__init__.py:58-109 take directly) at the price of one copy of each operand."""
+    D, Dv = query.shape[-1], value.shape[-1]
+    to = 64 if max(D, Dv) <= 64 else 128
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    pad = torch.nn.functional.pad
+    return pad(query, (0, to - D)), pad(key, (0, to - D)), pad(value, (0, to - Dv)), scale
+
+
+def _out_like(query, value=None):
     """The attention output for ``query``: the query's own memory layout (a [B,S,H,D]-memory view stays one, so the
     caller's transpose back is free) whenever the kernels can write it -- unit head_dim stride, 16-byte aligned rows
-    -- and contiguous otherwise.  Reads sizes and strides only, so the fake implementations allocate through it
-    too and a compiled graph is planned against the strides the kernel really writes."""
+    -- and contiguous otherwise (also for the head_dims that run zero-padded).  Reads sizes and strides only, so
+    the fake implementations allocate through it too and a compiled graph is planned against the strides the
+    kernel really writes."""
+    if value is not None and not _native_head_dims(query, value):
+        return torch.empty((*query.shape[:3], value.shape[-1]), dtype=query.dtype, device=query.device)
     out = torch.empty_like(query)
     if out.stride(-1) != 1 or any(out.shape[d] > 1 and out.stride(d) % 8 for d in range(out.ndim - 1)):
         out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
@@ -78,7 +100,7 @@ def _same_device(ref, **operands):
             raise ValueError(f"{name} is on {t.device} but must be on {ref.device}: all operands must share one device")
 
 
-def _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask=None, causal_ok=False):
+def _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask=None, causal_ok=False, any_head_dim=False):
     if query.ndim != 4 or key.ndim != 4 or value.ndim != 4:
         raise ValueError("query, key and value must be 4-D [batch, heads, seq, head_dim]")
     _same_device(query, key=key, value=value, attn_mask=attn_mask)
@@ -95,8 +117,12 @@ def _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask=None, ca
     B, H, Sq, D = query.shape
     if key.shape[0] != B or key.shape[1] != H or key.shape[3] != D:
         raise ValueError(f"key shape {tuple(key.shape)} does not match query {tuple(query.shape)}")
-    if value.shape[:3] != key.shape[:3] or value.shape[3] != D:
+    if value.shape[:3] != key.shape[:3]:
         raise ValueError(f"value shape {tuple(value.shape)} does not match key {tuple(key.shape)}")
+    if (value.shape[3] != D or D not in (64, 128)) and not any_head_dim:
+        raise NotImplementedError(f"head_dim {D} / value width {value.shape[3]}: this op takes 64 or 128 with values as wide as the keys")
+    if max(D, value.shape[3]) > 128 or min(D, value.shape[3]) < 1:
+        raise NotImplementedError(f"head_dim {D} / value width {value.shape[3]} not supported (1..128)")
 
 
 def _dense_forward(query, key, value, scale, want_lse, kv_len=None, is_causal=False):
@@ -184,6 +210,10 @@ def _masked_forward(query, key, value, attn_mask, scale, want_lse, is_causal=Fal
     """attn_mask / is_causal handling shared by the three SDPA-signature ops.  Nothing here reads the mask on
     the host: whether a key mask is a prefix is settled on the device (pa_attn_fwd_masked), so masked calls can
     be captured in a HIP graph like the unmasked ones."""
+    if not _native_head_dims(query, value):
+        q, k, v, scale = _pad_head_dims(query, key, value, scale)
+        out, lse = _masked_forward(q, k, v, attn_mask, scale, want_lse, is_causal)
+        return out[..., : value.shape[-1]].contiguous(), lse
     if attn_mask is None:
         return _dense_forward(query, key, value, scale, want_lse, is_causal=is_causal)
     B, H, Sq, D = query.shape
@@ -225,14 +255,14 @@ def attention_forward_with_lse(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """out [B,H,Sq,D] in query's dtype and natural-log LSE [B,H,Sq] in fp32
     (src/para_attn/ops/__init__.py:160-179)."""
-    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask, causal_ok=True)
+    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask, causal_ok=True, any_head_dim=True)
     out, lse = _masked_forward(query, key, value, attn_mask, scale, True, is_causal)
     return out, lse
 
 
 @torch.library.register_fake("para_attn::attention_forward_with_lse")
 def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
-    return _out_like(query), _lse_like(query)
+    return _out_like(query, value), _lse_like(query)
 
 
 @torch.library.custom_op("para_attn::attention_forward", mutates_args=(), device_types=("cuda",))
@@ -247,14 +277,14 @@ def attention_forward(
     scale: Optional[float] = None,
 ) -> torch.Tensor:
     """Plain SDPA forward, no LSE (src/para_attn/ops/__init__.py:204-223)."""
-    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask, causal_ok=True)
+    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask, causal_ok=True, any_head_dim=True)
     out, _ = _masked_forward(query, key, value, attn_mask, scale, False, is_causal)
     return out
 
 
 @torch.library.register_fake("para_attn::attention_forward")
 def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
-    return _out_like(query)
+    return _out_like(query, value)
 
 
 @torch.library.custom_op("para_attn::attention_forward_sparse_kv", mutates_args=(), device_types=("cuda",))
@@ -275,9 +305,9 @@ def attention_forward_sparse_kv(
     excludes is_causal (:270).  A prefix mask (valid text length) costs nothing:
     the kernel just stops at the per-batch key count.
     """
-    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask)
+    _check_sdpa_args(query, key, value, dropout_p, is_causal, attn_mask, any_head_dim=True)
     if attn_mask is None:
-        return _dense_forward(query, key, value, scale, False)[0]
+        return _masked_forward(query, key, value, None, scale, False)[0]
     if attn_mask.dtype != torch.bool:
         raise AssertionError("attn_mask must be a boolean tensor")
     m = attn_mask
@@ -293,7 +323,7 @@ def attention_forward_sparse_kv(
 
 @torch.library.register_fake("para_attn::attention_forward_sparse_kv")
 def _(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, *, scale=None):
-    return _out_like(query)
+    return _out_like(query, value)
 
 
 # ---------------------------------------------------------------------------------

@@ -533,6 +533,51 @@ def test_score_bound_at_the_limit(cuda, dtype, D, bm, side, tuning):
     assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("D,Dv", [(32, 32), (40, 40), (72, 72), (80, 80), (96, 96), (128, 64), (64, 128), (16, 24), (120, 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_other_head_dims(cuda, D, Dv, dtype):
+    """head_dims other than 64 and 128, and values narrower or wider than the keys, as aten's kernels behind the
+    reference's op take them (src/para_attn/ops/__init__.py:58-109): the default scale is that of the true head_dim,
+    out has the values' width, with and without a mask and is_causal; against the fp64 oracle and torch's CPU SDPA,
+    and through F.scaled_dot_product_attention under the mode."""
+    B, H, Sq, Skv = 2, 3, 150, 333
+    g = torch.Generator().manual_seed(D * 131 + Dv)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    k = torch.randn(B, H, Skv, D, generator=g).to(dtype)
+    v = torch.randn(B, H, Skv, Dv, generator=g).to(dtype)
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd)
+    assert out.shape == (B, H, Sq, Dv) and out.dtype == dtype and out.is_contiguous() and lse.shape == (B, H, Sq)
+    _check(out, lse, ref_out, ref_lse, f"head_dim {D}/{Dv} {dtype}")
+    if D == Dv:
+        cpu_out, cpu_lse = oattn.sdpa_lse_torch_cpu(q.float(), k.float(), v.float())
+        _check(out, lse, cpu_out.numpy(), cpu_lse.numpy(), f"head_dim {D}/{Dv} {dtype} vs torch CPU")
+    else:  # torch's CPU flash routine wants one head size; its composite SDPA takes any (no LSE from it)
+        cpu_out = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+        _check(out, None, cpu_out.numpy(), None, f"head_dim {D}/{Dv} {dtype} vs torch CPU")
+    assert torch.equal(torch.ops.para_attn.attention_forward(qd, kd, vd), out)
+    # a scale of the caller's, a key mask that is no prefix, is_causal
+    keep = torch.rand(B, 1, 1, Skv, generator=g) < 0.6
+    keep[..., 0] = True
+    m_out, m_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), 0.2, keep.numpy())
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, keep.to(cuda), scale=0.2)
+    _check(out, lse, m_out, m_lse, f"head_dim {D}/{Dv} masked")
+    assert torch.equal(torch.ops.para_attn.attention_forward_sparse_kv(qd, kd, vd, keep.to(cuda), scale=0.2), out)
+    c_out, c_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, oattn.causal_keep(Sq, Skv))
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, is_causal=True)
+    _check(out, lse, c_out, c_lse, f"head_dim {D}/{Dv} causal")
+    import paraattention_amd
+
+    with paraattention_amd.UnifiedAttnMode():
+        routed = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd)
+    assert torch.equal(routed, torch.ops.para_attn.attention_forward(qd, kd, vd))
+    torch.library.opcheck(torch.ops.para_attn.attention_forward_with_lse.default, (qd, kd, vd), test_utils="test_faketensor")
+    with pytest.raises(NotImplementedError):
+        torch.ops.para_attn.attention_forward(torch.zeros(1, 1, 4, 160, dtype=dtype, device=cuda), torch.zeros(1, 1, 4, 160, dtype=dtype, device=cuda),
+                                              torch.zeros(1, 1, 4, 160, dtype=dtype, device=cuda))
+
+
 CAUSAL = [(1, 2, 1, 1), (1, 1, 17, 17), (2, 2, 64, 64), (1, 2, 129, 129), (1, 1, 300, 300), (1, 2, 700, 700),
           (1, 1, 300, 90), (1, 2, 90, 300), (1, 1, 1000, 1000)]
 
