@@ -19,7 +19,7 @@ the gap), so the defaults warm every loop up for that long (30 calls of the head
 memory-side cache cannot hold a working set from one call to the next; a sample of rows of the last
 timed output of every attention shape is compared with torch's CPU SDPA (``checked``).
 
-``--only {attn,merge,fbcache,taylorseer,sparse,ring,flux,wan,shapes,copy,yardsticks}`` runs a single loop (what
+``--only {attn,merge,fbcache,taylorseer,sparse,ring,flux,wan,shapes,copy,yardsticks,wave_rows}`` runs a single loop (what
 the rocprofv3 summaries under profiles/ were taken with).
 """
 import argparse
@@ -38,8 +38,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Traffic at the L2's memory side per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two
 # rocprofv3 --pmc runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy).  These counters cannot be
 # read from inside this process; the figures are those of the summary named in TRAFFIC_SOURCE, not of this run.
-TRAFFIC = {"attn": 9.553e9, "merge": 4.771e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 1.893e10,
-           "flux": 3.06e8, "ring_sweep": 1.224e10, "ring_sweep_per_block": 1.509e10, "wan_self": 3.361e9, "wan_cross": 7.21e8}
+TRAFFIC = {"attn": 1.001e10, "merge": 4.772e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 1.923e10,
+           "flux": 3.15e8, "ring_sweep": 1.224e10, "ring_sweep_per_block": 1.509e10, "wan_self": 3.581e9, "wan_cross": 8.21e8,
+           "causal": 3.131e10, "head_dim_64": 2.438e9}
 TRAFFIC_SOURCE = "profiles/kernels_bench_workloads.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the same command)"
 
 
@@ -229,10 +230,49 @@ def bench_shapes(dev, steps=10, warmup=5):
     """Two further dense shapes: the headline shape with is_causal (flops of the kept half) and a head_dim 64 shape."""
     return {
         "headline_shape_causal": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=5,
-                                             check_heads=(0, 1), causal=True),
+                                             check_heads=(0, 1), causal=True, traffic="causal"),
         "head_dim_64": _dense_case(dev, "head_dim 64 (CogVideoX-like)", 1, 48, 17776, 17776, 64, steps, warmup, seed=6,
-                                   check_heads=(0, 23)),
+                                   check_heads=(0, 23), traffic="head_dim_64"),
     }
+
+
+def bench_wave_rows(dev, steps=12, warmup=20):
+    """The resident-workgroup kernel as 8 wavefronts of 32 query rows (what ships) against 4 wavefronts of 64 (knob
+    "wave_rows"), alternating twice in one process on the same tensors: median ms and fraction of the MFMA peak per
+    setting and shape.  The two forms give the same bits, which is checked."""
+    import statistics as st
+
+    import torch
+
+    from oracle import inputs
+    from paraattention_amd import _lib
+
+    op = torch.ops.para_attn.attention_forward_with_lse
+    out = {}
+    shapes = [("headline", 1, 3, 119056, 119056, True), ("wan_self", 1, 40, 32760, 32760, False),
+              ("ring_block", 1, 24, 14882, 14882, False), ("flux", 1, 24, 4608, 4608, False), ("wan_cross", 1, 40, 32760, 512, False)]
+    try:
+        for name, B, H, Sq, Skv, rms in shapes:
+            q, k, v = (t.to(dev) for t in inputs.qkv(B, H, Sq, Skv, 128, seed=0, rms_norm_qk=rms))
+            flops = 4.0 * B * H * Sq * Skv * 128
+            long = flops > 1e13
+            ref, rows = None, {32: [], 64: []}
+            for _ in range(2):
+                for wr in (32, 64):
+                    _lib.set_tuning("wave_rows", wr)
+                    t = _time_calls(lambda i: op(q, k, v), steps if long else 4 * steps, warmup if long else 5 * warmup)
+                    rows[wr].append(t["median"])
+                    o, l = op(q, k, v)
+                    if ref is None:
+                        ref = (o, l)
+                    elif not (torch.equal(o, ref[0]) and torch.equal(l, ref[1])):
+                        raise AssertionError(f"{name}: the two wavefront forms differ")
+            out[name] = {f"rows_{wr}": {"ms_median": round(st.median(ms), 4), "frac": round(flops / (st.median(ms) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+                         for wr, ms in rows.items()}
+            del q, k, v
+    finally:
+        _lib.set_tuning("wave_rows", 0)
+    return out
 
 
 def bench_sparse(dev, steps=10, warmup=10):
@@ -355,7 +395,7 @@ def bench_yardsticks(dev, steps=30, warmup=60):
     (bus turn-arounds), so a kernel that reads 6 bytes and writes 4 per element cannot be priced like one that
     only reads.  (1) torch's ``acc.add_(blk)`` on the merge step's operands: fp32 read + 16-bit read + fp32 write
     per element, the same bytes as the merge step less its LSE words, three buffer sets rotated; (2) a 1 GiB copy
-    (half reads, half writes); (3) a read-only pass (``sum`` over the fp32 accumulators)."""
+    (half reads, half writes).  The read-only end of the scale is the FBCache reduction (``--only fbcache``)."""
     import torch
 
     B, H, S, D = 1, 24, 14882, 128
@@ -366,8 +406,6 @@ def bench_yardsticks(dev, steps=30, warmup=60):
     t = _time_calls(lambda i: sets[i % SETS][0].add_(sets[i % SETS][1]), steps, warmup)
     out["add_fp32_bf16_in_place"] = _hbm("yardstick", "torch add_: fp32 [1,24,14882,128] += bf16, in place (6 B read, 4 B written per element)",
                                          B * H * S * D * 10, t, SETS)
-    t = _time_calls(lambda i: sets[i % SETS][0].sum(), steps, warmup)
-    out["sum_fp32_read_only"] = _hbm("yardstick", "torch sum over fp32 [1,24,14882,128] (reads only)", B * H * S * D * 4, t, SETS)
     del sets
     out["copy_1GiB"] = bench_copy(dev)
     return out
@@ -418,7 +456,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     singles = {"merge": bench_merge, "fbcache": bench_fbcache, "taylorseer": bench_taylorseer, "sparse": bench_sparse,
                "ring": bench_ring, "flux": bench_flux, "wan": bench_wan, "shapes": bench_shapes, "copy": bench_copy,
-               "yardsticks": bench_yardsticks}
+               "yardsticks": bench_yardsticks, "wave_rows": bench_wave_rows}
     ap.add_argument("--only", choices=["attn"] + list(singles), default=None,
                     help="profiling aid: run just one kernel's timed loop and print its figures")
     args = ap.parse_args()
@@ -465,7 +503,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "pa::attn_fwd_d128_stream_kernel<pa::BF16, true>",
+            "kernel": "pa::attn_fwd_d128_stream_kernel<pa::BF16, true, 1>",
             "achieved": round(kern_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",

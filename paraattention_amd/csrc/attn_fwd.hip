@@ -1797,6 +1797,51 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
   }
 }
 
+// Where the softmax of a score tile goes in an iteration of attn_fwd_d128_stream_kernel with 64 rows per wavefront
+// (see there): 170 small steps, step i in the gap behind MFMA gap[i] of the iteration, -1 for the steps that do
+// not exist (the first and last slots hold fewer).
+struct Rb2Steps {
+  static constexpr int N = 170;
+  int gap[N];
+  int lo[64], hi[64];  // the steps of gap q are lo[q] .. hi[q] - 1 (their gaps ascend), less those that do not exist
+  static constexpr int pair(int i) {
+    const int slot = i / 5, kind = i % 5;
+    return kind == 0 ? slot - 2 : kind < 3 ? slot - 1 : slot;
+  }
+  static constexpr int cost(int i) {
+    const int n = pair(i), kind = i % 5;
+    return n < 0 || n > 31 ? 0 : kind == 0 ? 12 : kind < 3 ? 8 : 12;
+  }
+  constexpr Rb2Steps() : gap() {
+    int total = 0;
+    for (int i = 0; i < N; ++i) total += cost(i);
+    int before = 0;
+    for (int i = 0; i < N; ++i) {
+      gap[i] = cost(i) == 0 ? -1 : (2 * before + cost(i)) * 30 / total;  // 60 gaps, by the middle of the step's span
+      before += cost(i);
+    }
+    for (int q = 0; q < 64; ++q) {
+      lo[q] = N;
+      hi[q] = 0;
+      for (int i = 0; i < N; ++i)
+        if (gap[i] == q) {
+          if (i < lo[q]) lo[q] = i;
+          hi[q] = i + 1;
+        }
+    }
+  }
+};
+constexpr Rb2Steps RB2_STEPS{};
+
+// every 16-key chunk of probabilities is packed before the PV MFMAs that take it: row block 0's before MFMA 32 + 8 k,
+// row block 1's before MFMA 36 + 8 k (step C of pair n is small step 5 (n + 2))
+constexpr bool rb2_steps_meet_deadlines() {
+  for (int k = 0; k < 4; ++k)
+    if (RB2_STEPS.gap[5 * (8 * k + 3 + 2)] >= 32 + 8 * k || RB2_STEPS.gap[5 * (8 * k + 7 + 2)] >= 36 + 8 * k) return false;
+  return true;
+}
+static_assert(rb2_steps_meet_deadlines(), "softmax steps are dealt too late for the second GEMM");
+
 // ---------------------------------------------------------------------------------------------
 // head_dim 128, resident workgroups (StreamPlan above): the two-tile pipeline of
 // attn_fwd_d128_pipe_kernel<.., 8> run over a list of pieces per workgroup as ONE stream of key
@@ -1807,6 +1852,15 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
 // stored from inside the loop.  What a launch of one workgroup per piece pays per piece (Q load,
 // first copies, S(0), output drain: 5-10 us against 1.7 us per key tile) is hidden behind the
 // neighbouring pieces' MFMA work.  Dense, not causal, no per-batch key counts.
+//
+// RB = query row blocks of 32 per wavefront.  RB = 1: 8 wavefronts of 32 rows, two per SIMD, everything in
+// the 256 vector registers a wavefront then has (the form that ships).  RB = 2: 4 wavefronts of 64 rows, one per
+// SIMD with 512 registers (the output and score accumulators in accumulation registers); every fragment read
+// from LDS feeds two MFMAs, so the workgroup reads half the LDS bytes per flop, but the scores have to be
+// read back from the accumulation registers (one more vector instruction per score) and one wavefront has to
+// overlap its softmax with its own MFMAs.  Same results bit for bit; measured at the same speed as RB = 1 on
+// the long shapes (the kernel sits at the chip's power limit either way: 68 % MFMA occupancy at 1.72 GHz
+// against 74 % at 1.60 GHz) and slower on short pieces, so it stays behind the "wave_rows" knob.
 // ---------------------------------------------------------------------------------------------
 template <typename T, bool BOUNDED, int RB = 1>
 __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const AttnParams p) {
@@ -2165,7 +2219,9 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   };
 
   vec8 f[8];          // ring of 8 operand fragments
-  floatx16 sn[RB][2];  // S(j+1) per row block (keys 0..31, 32..63)
+  // S(j+1) per row block (keys 0..31, 32..63); with 64 rows per wavefront two sets that alternate by the iteration's parity
+  floatx16 sbuf[RB][RB][2];
+  floatx16 (&sn)[RB][2] = sbuf[0];
   float mx[RB];        // row maximum of S(j), masked, unscaled
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -2343,14 +2399,13 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
       // ---- 64 query rows per wavefront, one wavefront per SIMD ------------------------------------------
       // Every K and V^T fragment read from LDS feeds two MFMAs (one per row block), so the workgroup reads half
       // the LDS bytes per flop of the 32-row form.  No second wavefront shares the SIMD: the softmax of S(j) has
-      // to run under this wavefront's own MFMAs, spread evenly over both GEMMs (34 slots under MFMAs 0..59 of
-      // the iteration's 64), each group of 16 probabilities finished just before the PV MFMAs that take it.
-      floatx16 cs[RB][2];  // S(j)
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        cs[rb][0] = sn[rb][0];
-        cs[rb][1] = sn[rb][1];
-      }
+      // to run under this wavefront's own MFMAs, a few instructions behind each of them (an MFMA leaves about 20
+      // of its 32 clocks to other vector instructions of the same wavefront), spread evenly over both GEMMs, each
+      // group of 16 probabilities finished just before the PV MFMAs that take it.  The score tiles live in
+      // accumulation registers; two sets alternate by the iteration's parity, S(j) is read from one pair by pair
+      // where the softmax takes it while S(j+1) gathers in the other, and no copy of a whole tile is made.
+      floatx16 (&cs)[RB][2] = sbuf[par];      // S(j)
+      floatx16 (&sn)[RB][2] = sbuf[par ^ 1];  // S(j+1)
 
       __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
@@ -2378,37 +2433,43 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
 
       // Softmax of S(j) in 32 pairs of scores, in the order the second GEMM takes them: pair n belongs to the
       // 16-key chunk n / 8 (key half t = n / 16, chunk cc of it), row block (n / 4) % 2, registers 8 cc + 2 (n % 4).
-      // A pair passes three slots: scale, exponentials, sum + pack.
+      // A pair passes three steps -- scale (A), exponentials (B), sum + pack (C), the first two one score at a time
+      // -- and the steps of consecutive pairs interleave as C(n-2), B(n-1), A(n); that sequence of 160 small steps
+      // is dealt out to the gaps behind the iteration's MFMAs by its running cost in clocks, so every gap holds
+      // about the same amount of it.
       uint32_t pk[RB][2][8];
       float lsum[RB];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) lsum[rb] = 0.f;
       float tf[2][2], te[2][2];
-      auto expo_slot = [&](int n) __attribute__((always_inline)) {
-        if (n >= 2 && n < 34) {
-          const int j = n - 2, rb = (j >> 2) & 1, k = j >> 3;
-          lsum[rb] += te[j & 1][0] + te[j & 1][1];
-          asm volatile("" : "+v"(lsum[rb]));
-          pk[rb][k >> 1][4 * (k & 1) + (j & 3)] = T::pack2(te[j & 1][0], te[j & 1][1]);
-        }
-        if (n >= 1 && n < 33) {
-          const int j = n - 1;
-          te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
-          te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
-        }
-        if (n < 32) {
-          const int rb = (n >> 2) & 1, k = n >> 3;
-          const floatx16& src = cs[rb][k >> 1];
-          const int r0 = 8 * (k & 1) + 2 * (n & 3);
-          tf[n & 1][0] = __builtin_fmaf(src[r0], c, -m_run[rb]);
-          tf[n & 1][1] = __builtin_fmaf(src[r0 + 1], c, -m_run[rb]);
-        }
+      auto step_a = [&](int n, int x) __attribute__((always_inline)) {
+        const int rb = (n >> 2) & 1, k = n >> 3;
+        const floatx16& src = cs[rb][k >> 1];
+        const int r0 = 8 * (k & 1) + 2 * (n & 3);
+        tf[n & 1][x] = __builtin_fmaf(src[r0 + x], c, -m_run[rb]);
       };
-      // slots finished once MFMA q of the iteration has been issued
-      auto slots_done = [](int q) constexpr { return q < 0 ? 0 : ((q + 1) * 34 / 60 < 34 ? (q + 1) * 34 / 60 : 34); };
-      auto run_slots = [&](int q) __attribute__((always_inline)) {
+      auto step_b = [&](int n, int x) __attribute__((always_inline)) {
+        te[n & 1][x] = __builtin_amdgcn_exp2f(tf[n & 1][x]);
+      };
+      auto step_c = [&](int n) __attribute__((always_inline)) {
+        const int rb = (n >> 2) & 1, k = n >> 3;
+        lsum[rb] += te[n & 1][0] + te[n & 1][1];
+        asm volatile("" : "+v"(lsum[rb]));
+        pk[rb][k >> 1][4 * (k & 1) + (n & 3)] = T::pack2(te[n & 1][0], te[n & 1][1]);
+      };
+      // small steps i = 0..169: slot i / 5 holds C(slot - 2), B(slot - 1) twice, A(slot) twice; their clocks: 12, 8, 8,
+      // 12, 12 (A: a read of an accumulation register and a multiplication) -- 52 per pair, 1664 in all, dealt to
+      // gaps 0..59 by the middle of each step's span (Rb2Steps, worked out at compile time)
+      auto run_steps = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
-        for (int n = slots_done(q - 1); n < slots_done(q); ++n) expo_slot(n);
+        for (int i = RB2_STEPS.lo[q]; i < RB2_STEPS.hi[q]; ++i) {
+          if (RB2_STEPS.gap[i] == q) {
+            const int kind = i % 5, n = Rb2Steps::pair(i);
+            if (kind == 0) step_c(n);
+            else if (kind < 3) step_b(n, kind - 1);
+            else step_a(n, kind - 3);
+          }
+        }
       };
 
       // ---- S(j+1) = K(j+1) Q^T: 32 MFMAs; the copies of K(j+2) and V(j+1) behind the first eight -------
@@ -2425,7 +2486,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
           if (q < IPW) dma_k1(par, nx2.n0, q, inside);
           else if (q < 2 * IPW) dma_v1(par ^ 1, nxt.n0, q - IPW, inside);
           if (rb == RB - 1) f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
-          run_slots(q);
+          run_steps(q);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -2436,7 +2497,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
           const int q = 16 + 2 * g + rb;
           sn[rb][g & 1] = T::mfma32(f[g], qf[rb][4 + (g >> 1)], sn[rb][g & 1]);
           if (rb == RB - 1) f[g] = read_vt(tV, 0, g >> 2, g & 3);
-          run_slots(q);
+          run_steps(q);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -2470,7 +2531,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
               const int g = cc * 4 + db;
               o[rb][db] = T::mfma32(f[g], bfrag, o[rb][db]);
               if (t == 0 && rb == RB - 1) f[g] = read_vt(tV, 1, cc, db);
-              run_slots(32 + u);
+              run_steps(32 + u);
               if constexpr (!BOUNDED) {
                 const floatx16& sx = sn[u >> 4][(u >> 3) & 1];
                 const int i = u & 7;
