@@ -707,7 +707,10 @@ def test_unsupported_raise(cuda):
     q, k, v = (t.to(cuda) for t in inputs.qkv(1, 1, 16, 16, 128))
     with pytest.raises(NotImplementedError):
         torch.ops.para_attn.attention_forward_with_lse(q, k, v, dropout_p=0.1)
-    with pytest.raises(NotImplementedError):
-        torch.ops.para_attn.attention_forward_with_lse(q[..., :32], k[..., :32], v[..., :32])
+    big = torch.zeros(1, 1, 16, 160, dtype=q.dtype, device=cuda)
+    with pytest.raises(NotImplementedError):  # head_dim above 128 (up to 128 runs, zero-padded where it is not 64 or 128)
+        torch.ops.para_attn.attention_forward_with_lse(big, big, big)
+    with pytest.raises(NotImplementedError):  # the ops outside the SDPA signature take 64 / 128 only
+        torch.ops.para_attn.attention_forward_sweep(q[..., :32], [k[..., :32]], [v[..., :32]])
     with pytest.raises(NotImplementedError):
         torch.ops.para_attn.attention_forward_with_lse(q.float(), k.float(), v.float())
