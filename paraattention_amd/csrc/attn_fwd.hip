@@ -1812,7 +1812,7 @@ struct Rb2Steps {
     const int n = pair(i), kind = i % 5;
     return n < 0 || n > 31 ? 0 : kind == 0 ? 12 : kind < 3 ? 8 : 12;
   }
-  constexpr Rb2Steps() : gap() {
+  constexpr Rb2Steps() : gap(), lo(), hi() {
     int total = 0;
     for (int i = 0; i < N; ++i) total += cost(i);
     int before = 0;
