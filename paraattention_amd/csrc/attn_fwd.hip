@@ -2719,9 +2719,9 @@ __global__ __launch_bounds__(256) void attn_split_merge_kernel(const AttnParams 
 }
 
 // Turns a [Hm,nQ,nK] block mask into per-segment lists of key ranges.
-// One wavefront per (hm, segment): the lanes read 64 mask bytes at a time and vote them into a
-// bit word; lane 0 then walks the words and emits the runs of kept blocks (the scan of
-// src/para_attn/sparse_attn.py:215-234), merged with the dense key margins where they touch.
+// One wavefront per (hm, segment): the lanes look at 64 key blocks at a time, vote where runs of kept
+// blocks begin and end, and each beginning / ending lane writes its bound of its range (the runs the
+// scan of src/para_attn/sparse_attn.py:215-234 finds), merged with the dense key margins where they touch.
 // Segments 0 and nQ+1 are the dense query margins.
 __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK,
                                                         int Skv, int kv_lo, int kv_block, int cap,
@@ -2745,57 +2745,41 @@ __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int
   }
   const uint8_t* row = mask + ((size_t)hm * nQ + (seg - 1)) * nK;
   const int kv_hi = kv_lo + nK * kv_block;
-  int n = 0;
-  int cur_b = -1, cur_e = -1;  // open range (lane 0 only)
-  auto push = [&](int b, int e) {
-    if (e <= b) return;
-    if (cur_e == b) {
-      cur_e = e;  // touches the open range: extend it
-    } else {
-      if (cur_e > cur_b) {
-        rg[2 * n] = cur_b;
-        rg[2 * n + 1] = cur_e;
-        ++n;
-      }
-      cur_b = b;
-      cur_e = e;
-    }
-  };
-  if (lane == 0) push(0, kv_lo);
-  int run_start = -1;  // block index where the current run of kept blocks began, -1 = none
+  // Every lane looks at one key block per pass: a run begins at a kept block whose left neighbour is dropped and
+  // ends at a kept block whose right neighbour is dropped; the k-th begin and the k-th end (counted with ballots
+  // and a running total) belong to range k.  The dense margins [0, kv_lo) and [kv_hi, Skv) join the first / last
+  // run where block 0 / block nK - 1 is kept, and stand as ranges of their own otherwise.
+  const bool left = kv_lo > 0, right = Skv > kv_hi;
+  const bool first_kept = row[0] != 0, last_kept = row[nK - 1] != 0;
+  const int first_idx = left && !first_kept ? 1 : 0;  // range index of the first run
+  int begins = 0, ends = 0;                           // runs begun / ended in the passes so far
+  const uint64_t below = lane == 0 ? 0 : (~0ull >> (64 - lane));
   for (int base = 0; base < nK; base += 64) {
     const int j = base + lane;
     const bool keep = j < nK && row[j] != 0;
-    uint64_t bits = __ballot(keep);
-    if (lane == 0) {
-      int pos = 0;  // bits below pos are consumed
-      while (pos < 64) {
-        if (run_start < 0) {
-          if (bits == 0) break;
-          const int z = __builtin_ctzll(bits);  // skip dropped blocks
-          pos += z;
-          bits >>= z;  // z <= 63 because bits != 0
-          run_start = base + pos;
-        } else {
-          const uint64_t inv = ~bits;
-          const int o = inv == 0 ? 64 : __builtin_ctzll(inv);
-          const int ones = o < 64 - pos ? o : 64 - pos;  // kept blocks in a row, within this word
-          pos += ones;
-          bits = ones < 64 ? bits >> ones : 0;
-          if (pos < 64) {  // the run ended inside this word
-            push(kv_lo + run_start * kv_block, kv_lo + (base + pos) * kv_block);
-            run_start = -1;
-          }
-        }
-      }
+    const bool begin = keep && (j == 0 || row[j - 1] == 0);
+    const bool end = keep && (j == nK - 1 || row[j + 1] == 0);
+    const uint64_t bb = __ballot(begin), eb = __ballot(end);
+    if (begin) {
+      const int k = begins + __builtin_popcountll(bb & below);
+      rg[2 * (first_idx + k)] = (j == 0 && left) ? 0 : kv_lo + j * kv_block;
     }
+    if (end) {
+      const int k = ends + __builtin_popcountll(eb & below);
+      rg[2 * (first_idx + k) + 1] = (j == nK - 1 && right) ? Skv : kv_lo + (j + 1) * kv_block;
+    }
+    begins += __builtin_popcountll(bb);
+    ends += __builtin_popcountll(eb);
   }
   if (lane == 0) {
-    if (run_start >= 0) push(kv_lo + run_start * kv_block, kv_hi);
-    push(kv_hi, Skv);
-    if (cur_e > cur_b) {
-      rg[2 * n] = cur_b;
-      rg[2 * n + 1] = cur_e;
+    int n = first_idx + begins;
+    if (left && !first_kept) {
+      rg[0] = 0;
+      rg[1] = kv_lo;
+    }
+    if (right && !last_kept) {
+      rg[2 * n] = kv_hi;
+      rg[2 * n + 1] = Skv;
       ++n;
     }
     *cnt = n;
