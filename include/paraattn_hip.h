@@ -292,7 +292,7 @@ PA_API int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int nQ, 
  * step of a pipeline under the reference's StructSparseAttnMode,
  * src/para_attn/sparse_attn.py:643-677, uses one mask): `runs` is what
  * pa_blocksparse_build_runs wrote for the same Hm, nQ, nK, Skv, kv_lo and
- * kv_block, and is only read here, so the run extraction (about 50 us at a
+ * kv_block, and is only read here, so the run extraction (about 9 us at a
  * [24,256,256] mask) is paid once.  The kernels cut every range at Skv and
  * end a walk at the first range beyond it, so a buffer built for a longer
  * key sequence cannot lead them past the tensors; ranges must be ascending
