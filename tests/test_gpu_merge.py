@@ -113,13 +113,15 @@ def test_ring_sweep_equals_full_attention(cuda, fused):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_one_launch_sweep(cuda, dtype, tuning):
+@pytest.mark.parametrize("wave_rows", [32, 64])
+def test_one_launch_sweep(cuda, dtype, wave_rows, tuning):
     """attention_forward_sweep: blocks at separate addresses walked as one key sequence.  Ragged block length
     (tiles never straddle blocks), ragged query length, [B,S,H,D] memory, 1 to 16 blocks, more pieces than the
     chip has compute units and fewer, with and without the score bound; against the fp64 oracle over the
     concatenated keys and bit for bit against the dense op on the concatenation where both take the same path."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     D = 128
+    tuning("wave_rows", wave_rows)  # both forms of the resident-workgroup kernel walk the segments
     for B, H, Sq, blk, n, bound in [(1, 2, 300, 290, 8, -1), (2, 3, 77, 64, 3, -1), (1, 4, 600, 1000, 16, 1), (1, 1, 256, 37, 1, -1),
                                     (1, 2, (cus // 2 + 3) * 256 - 100, 150, 4, 1)]:
         tuning("bound", bound)
@@ -143,12 +145,14 @@ def test_one_launch_sweep(cuda, dtype, tuning):
         torch.ops.para_attn.attention_forward_sweep(qd, kb, vb[:-1])
 
 
-def test_fused_accumulate_steps(cuda, tuning):
+@pytest.mark.parametrize("wave_rows", [32, 64])
+def test_fused_accumulate_steps(cuda, wave_rows, tuning):
     """attention_forward_accumulate_ / _final against the oracle's merge of the oracle's partials, on a grid that
     takes the key-split tail (so the split merge folds the accumulator too), with a strided query."""
     from oracle import merge as omerge
     from paraattention_amd import _lib
 
+    tuning("wave_rows", wave_rows)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     B, H, D = 1, 8, 128
     Sq = (cus // (B * H) + 3) * 256 - 77
