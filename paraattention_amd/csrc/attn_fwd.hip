@@ -2116,6 +2116,12 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
     const KArgs kp = kargs();
     const Where w = where(kp, d.piece);
     float* const acc_out = kp->acc_out;
+    // The addresses below are worked out here, from a lane number the compiler cannot see through.  Derived from
+    // `lane` they are loop invariants: two dozen registers held across the hot loop, spilled, and fetched back one
+    // by one between the output stores -- and a fetch from scratch memory waits for every store issued before it.
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int l32 = ln & 31, hh = ln >> 5, lane = ln;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       float l_tot;
@@ -2149,7 +2155,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
         for (int i = 0; i < 8; ++i) {
           const int r = 4 * i + (lane >> 4), ch = lane & 15;
           const u32x4 x = *(const u32x4*)(st + r * 256 + 16 * (ch ^ (r & 15)));
-          if (row0 + r < w.row_end) *(u32x4*)(obase + (int64_t)(row0 + r) * os_s + 8 * ch) = x;
+          if (row0 + r < w.row_end) __builtin_nontemporal_store(x, (u32x4*)(obase + (int64_t)(row0 + r) * os_s + 8 * ch));
         }
         float* const lse_out = kp->lse;
         if (lse_out != nullptr && hh == 0 && my_row < w.row_end)
@@ -2596,6 +2602,416 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
     tile_step(odd, std::false_type{});
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // no tile copy may still be on its way to LDS when the wavefront ends
+}
+
+// ---------------------------------------------------------------------------------------------
+// head_dim 128, 449..512 keys per (batch, head): cross-attention of many query rows to a short text.
+// A piece (256 query rows of one head) lives for eight key tiles only, so what happens once per piece -- its Q
+// rows coming in, its output going out -- decides the speed; attn_fwd_d128_stream_kernel pays for both in every
+// wavefront at the same time, in front of a workgroup barrier.  Here the key tiles of a head go round in a
+// circle (step s copies tile s mod 8; softmax does not care where in the circle a row begins), and the two
+// wavefronts of a SIMD are half a circle apart: wavefronts 0..3 begin their pieces at tile 0, wavefronts 4..7
+// at tile 4, so while one of a SIMD's two wavefronts changes pieces the other is in mid-piece and keeps the
+// matrix cores busy.  The half that is in mid-piece also issues all the tile copies; the half that changes
+// pieces issues none for four steps and therefore never waits at a barrier for its own loads and stores (one
+// counter covers tile copies, Q loads and output stores): its next Q rows travel into the wavefront's own 8 KB
+// of LDS a step and a half before they are needed, and its output leaves through the same 8 KB.
+// Workgroup g takes the pieces [g P / G, (g + 1) P / G); consecutive pieces of one head form a run of
+// 8 n + 4 steps (wavefronts 4..7 idle for the first four, 0..3 for the last four).
+// Dense, not causal, no per-batch key counts, no accumulation.
+// ---------------------------------------------------------------------------------------------
+constexpr int SHORT_NT = 8;  // key tiles of a piece
+constexpr int SHORT_QI = 5;  // step of a piece (0..7) at whose start the next piece's Q rows are sent for
+
+template <typename T>
+__global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnParams p) {
+  typedef typename T::vec8 vec8;
+  constexpr int DC = 8, DB = 4, NT = SHORT_NT, QI = SHORT_QI;
+  if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  char* const sK = (char*)smem;                   // [2][64][256 B]
+  char* const sV = (char*)smem + 2 * TILE_BYTES;  // [2][64][256 B]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  char* const sMine = (char*)smem + 4 * TILE_BYTES + wave * 8192;  // [32 rows][256 B]: Q on its way in, output on its way out
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+  const int phase = wave >> 2;  // 0: pieces begin at tile 0; 1: at tile 4
+  const int cw = wave & 3;      // this wavefront's share of a tile copy
+  const int G = p.st.G, P = p.st.n_pieces;
+  const int wg = p.st.xcd_order ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  int piece0 = (int)((int64_t)wg * P / G);
+  const int piece_end = (int)((int64_t)(wg + 1) * P / G);
+  if (piece0 >= piece_end) return;  // before any barrier: the whole workgroup leaves
+
+  auto lds_barrier = [&]() __attribute__((always_inline)) {  // orders LDS traffic only: loads and stores to memory stay in flight
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  };
+  auto wait_vm = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+
+  // ---- global -> LDS copies: 4 wavefronts move a tile, 4 instructions each -----------------------
+  const uint32_t ks_bytes = (uint32_t)(p.ks_s * 2), vs_bytes = (uint32_t)(p.vs_s * 2), qs_bytes = (uint32_t)(p.qs_s * 2);
+  auto make_rsrc = [&](const void* base, uint64_t nbytes) __attribute__((always_inline)) {
+    const uint64_t a = (uint64_t)base;
+    u32x4 r;
+    r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+    r[2] = __builtin_amdgcn_readfirstlane((uint32_t)nbytes);
+    r[3] = 0x00020000u;
+    return r;
+  };
+  u32x4 krs = {0, 0, 0, 0x00020000u}, vrs = krs, qrs = krs, ors = krs;
+  const uint32_t os_bytes = (uint32_t)(p.os_s * 2);
+  const int dma_row = 4 * cw + (lane >> 4);
+  const int dma_pc = lane & 15;
+  const uint32_t k_off0 = dma_row * ks_bytes + 16 * (dma_pc ^ (dma_row & 15));
+  const uint32_t v_off0 = dma_row * vs_bytes + 16 * (dma_pc ^ (4 * (dma_row & 3)));
+  const uint32_t lds_k = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sK + cw * 1024);
+  const uint32_t lds_v = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sV + cw * 1024);
+  const uint32_t lds_mine = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_char*)sMine);
+  // instruction i of 4: rows 16 i + 4 cw .. + 3 of tile `tile` of the head
+  auto dma_k1 = [&](int buf, int tile, int i) __attribute__((always_inline)) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane((uint32_t)(tile * BN + 16 * i) * ks_bytes);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_k + buf * TILE_BYTES + i * 4096), "v"(k_off0), "s"(krs), "s"(soff) : "memory");
+  };
+  auto dma_v1 = [&](int buf, int tile, int i) __attribute__((always_inline)) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane((uint32_t)(tile * BN + 16 * i) * vs_bytes);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_v + buf * TILE_BYTES + i * 4096), "v"(v_off0), "s"(vrs), "s"(soff) : "memory");
+  };
+  // this wavefront's 32 query rows from row0 on -> its own 8 KB, 16-byte chunks XOR-swizzled by the row as in a K tile
+  // (rows past the last query row of the head lie outside the descriptor and arrive as zeros)
+  auto dma_q = [&](int row0) __attribute__((always_inline)) {
+    const uint32_t soff = __builtin_amdgcn_readfirstlane((uint32_t)row0 * qs_bytes);
+    int lane = tid & 63;  // the eight offsets are worked out here, not held across the loop
+    asm volatile("" : "+v"(lane));
+    const int dma_pc = lane & 15;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int rr = 4 * i + (lane >> 4);
+      const uint32_t voff = rr * qs_bytes + 16 * (dma_pc ^ (rr & 15));
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                   :: "s"(lds_mine + i * 1024), "v"(voff), "s"(qrs), "s"(soff) : "memory");
+    }
+  };
+
+  // ---- fragment read addresses (as in attn_fwd_d128_pipe_kernel) ------------------------------------
+  uint32_t ka[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) ka[dc] = l32 * 256 + 16 * ((2 * dc + hh) ^ (l32 & 15));
+  uint32_t va[DB];
+  {
+    const int g16 = lane >> 4, lg = lane & 15, r = lg >> 2, cq = lg & 3, dhalf = g16 & 1;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      va[db] = (4 * hh + r) * 256 + 16 * ((4 * db + 2 * dhalf + (cq >> 1)) ^ (4 * r)) + 8 * (cq & 1);
+  }
+  auto read_k = [&](const char* tile, int t, int dc) __attribute__((always_inline)) -> vec8 {
+    return *(const vec8*)(tile + t * 32 * 256 + ka[dc]);
+  };
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  auto read_vt = [&](const char* tile, int t, int c, int db) __attribute__((always_inline)) -> vec8 {
+    const char* a = tile + (32 * t + 16 * c) * 256 + va[db];
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + 8 * 256));
+    typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
+    s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(vec8, v);
+  };
+
+  vec8 qf[DC];  // B operand of the first GEMM
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) qf[dc] = __builtin_bit_cast(vec8, (u32x4){0u, 0u, 0u, 0u});
+  auto read_q = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) qf[dc] = *(const vec8*)(sMine + ka[dc]);
+  };
+
+  floatx16 o[DB];
+  float m_run = -INFINITY, l_run = 0.f;
+  auto reset_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+    m_run = -INFINITY;
+    l_run = 0.f;
+  };
+  const float c = p.scale_log2;
+  const int nv_last = p.Skv - (NT - 1) * BN;  // keys of tile 7: 1..64
+  const bool ragged = nv_last < BN;
+
+  auto mask_tail = [&](floatx16& a0, floatx16& a1, int nvalid) __attribute__((always_inline)) {
+    const int lim = nvalid - 4 * hh;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (8 * (r >> 2) + (r & 3) >= lim) a0[r] = -INFINITY;
+      if (8 * (r >> 2) + (r & 3) + 32 >= lim) a1[r] = -INFINITY;
+    }
+  };
+  auto across = [&](float x) __attribute__((always_inline)) {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+  };
+
+  vec8 f[8];          // ring of 8 operand fragments
+  floatx16 sn0, sn1;  // S(s+1): keys 0..31, 32..63 of the tile
+  float mx = 0.f;     // row maximum of S(s), masked, unscaled
+
+  while (piece0 < piece_end) {
+    // ---- a run of n consecutive pieces of one (batch, head) -----------------------------------------
+    const int nqt = p.n_qtiles;
+    const int bh = piece0 / nqt, qt0 = piece0 - bh * nqt;
+    const int n = piece_end - piece0 < nqt - qt0 ? piece_end - piece0 : nqt - qt0;
+    const int batch = bh / p.H, head = bh - batch * p.H;
+    const int steps = NT * n + NT / 2;
+    krs = make_rsrc((const uint16_t*)p.k + batch * p.ks_b + head * p.ks_h, (uint64_t)(p.Skv - 1) * ks_bytes + 256);
+    vrs = make_rsrc((const uint16_t*)p.v + batch * p.vs_b + head * p.vs_h, (uint64_t)(p.Skv - 1) * vs_bytes + 256);
+    qrs = make_rsrc((const uint16_t*)p.q + batch * p.qs_b + head * p.qs_h, (uint64_t)(p.Sq - 1) * qs_bytes + 256);
+    ors = make_rsrc((const uint16_t*)p.out + batch * p.os_b + head * p.os_h, (uint64_t)(p.Sq - 1) * os_bytes + 256);
+    auto row_of = [&](int k) __attribute__((always_inline)) { return (qt0 + k) * 256 + 32 * wave; };  // this wavefront's first row of piece k of the run
+
+    // A finished piece leaves in two parts, each at the end of a step, where the wavefront that changes pieces (it has
+    // priority over the other wavefront of its SIMD from step QI of a piece to step 0 of the next) would otherwise
+    // wait at the barrier: behind the piece's last step the accumulators are scaled, packed and staged in the
+    // wavefront's 8 KB, so that the data can leave as whole 256-byte rows, four per instruction; behind the next
+    // piece's first step the rows are stored.  Addresses come from a lane number the compiler cannot see through
+    // (see finish_item of attn_fwd_d128_stream_kernel).
+    float lse_kept = 0.f;
+    auto finish_stage = [&]() __attribute__((always_inline)) {
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
+      const int l32 = ln & 31, hh = ln >> 5;
+      float l_tot;
+      {
+        auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+        l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+      }
+      const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+      lse_kept = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          u32x2 x;
+          x[0] = T::pack2(o[db][4 * a] * inv, o[db][4 * a + 1] * inv);
+          x[1] = T::pack2(o[db][4 * a + 2] * inv, o[db][4 * a + 3] * inv);
+          *(u32x2*)(sMine + l32 * 256 + 16 * ((4 * db + a) ^ (l32 & 15)) + 8 * hh) = x;
+        }
+    };
+    auto finish_store = [&](int k) __attribute__((always_inline)) {
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
+      const int l32 = ln & 31, hh = ln >> 5;
+      const int row0 = row_of(k);
+      // eight stores of four rows each through the output's descriptor: a row past the head's last query row lies
+      // outside it and is dropped, so the sequence needs no branch.  Non-temporal: nothing here reads the output
+      // again, and the launch runs at the chip's power limit, where the hint is worth 2.5 % of the time.
+      const int lr = ln >> 4, ch = ln & 15;
+      u32x4 x[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = *(const u32x4*)(sMine + (4 * i + lr) * 256 + 16 * (ch ^ ((4 * i + lr) & 15)));
+      const uint32_t voff = lr * os_bytes + 16 * ch;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t soff = __builtin_amdgcn_readfirstlane((uint32_t)(row0 + 4 * i) * os_bytes);
+        asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen nt" :: "v"(x[i]), "v"(voff), "s"(ors), "s"(soff) : "memory");
+      }
+      float* const lse_out = p.lse;
+      if (lse_out != nullptr && hh == 0 && row0 + l32 < p.Sq)
+        lse_out[((int64_t)batch * p.H + head) * p.Sq + row0 + l32] = lse_kept;
+    };
+
+    // ---- start of the run: wavefronts 4..7 (idle for four steps) copy K(0), V(0), K(1); 0..3 fetch their Q --------
+    wait_vm();
+    lds_barrier();  // nobody still reads the tiles of the run before
+    if (phase == 1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dma_k1(0, 0, i);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dma_v1(0, 0, i);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dma_k1(1, 1, i);
+    } else {
+      dma_q(row_of(0));
+    }
+    wait_vm();
+    lds_barrier();
+    if (phase == 0) read_q();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sn0[r] = sn1[r] = 0.f;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(sK, 0, dc);
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+      sn0 = T::mfma32(f[dc], qf[dc], sn0);
+      f[dc] = read_k(sK, 1, dc);
+    }
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) sn1 = T::mfma32(f[dc], qf[dc], sn1);
+    {
+      float m2 = fmaxf(sn0[0], sn1[0]);
+#pragma unroll
+      for (int r = 1; r < 16; ++r) m2 = fmaxf(fmaxf(m2, sn0[r]), sn1[r]);
+      mx = across(m2);
+    }
+    reset_acc();
+
+    // One step; PAR = s & 1 = buffer of tile s (K(s+1) sits in the other K buffer).
+    auto step = [&](auto PAR, int s) __attribute__((always_inline)) {
+      constexpr int par = decltype(PAR)::value;
+      const char* tV = sV + par * TILE_BYTES;
+      const char* tKn = sK + (par ^ 1) * TILE_BYTES;
+      const int rel = s - (NT / 2) * phase;
+      const int r = rel & (NT - 1);   // step of this wavefront's piece
+      const int k = rel >> 3;         // its piece of the run (-1: not yet; n: no more)
+      const bool copier = ((r - QI) & 7) >= 4;
+      const bool was_copier = ((r - 1 - QI) & 7) >= 4;
+      floatx16 c0 = sn0, c1 = sn1;  // S(s)
+
+      if (was_copier) wait_vm();  // the tile copies this wavefront issued in the step before have landed
+      lds_barrier();
+      // Of a SIMD's two wavefronts the older one (0..3) wins every arbitration and reaches the next barrier about a
+      // thousand clocks before the other.  The one that changes pieces in this step or the next has more to do, so
+      // it is given that lead.
+      if (r == QI) __builtin_amdgcn_s_setprio(2);
+      if (r == 1) __builtin_amdgcn_s_setprio(0);
+      if (r == QI && k + 1 < n) dma_q(row_of(k + 1));
+
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
+
+      {
+        const float mx_s = mx * c;
+        if (r == 0) {
+          m_run = mx_s;  // a piece's first tile: the accumulators hold nothing yet, so there is nothing to rescale
+        } else if (__any(mx_s > m_run + RESCALE_SLACK)) {
+          const float m_new = fmaxf(m_run, mx_s);
+          const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+          l_run *= alpha;
+#pragma unroll
+          for (int i = 0; i < DB; ++i)
+#pragma unroll
+            for (int r2 = 0; r2 < 16; ++r2) o[i][r2] *= alpha;
+          m_run = m_new;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- stage A: S(s+1) = K(s+1) Q^T, the copies of K(s+2) and V(s+1) --------------------------
+      uint32_t pk0[8], pk1[8];
+      float lsum = 0.f;
+      float tf[2][2], te[2][2];
+      auto expo_slot = [&](int nn) __attribute__((always_inline)) {
+        if (nn >= 2 && nn < 18) {
+          const int j = nn - 2;
+          lsum += te[j & 1][0] + te[j & 1][1];
+          asm volatile("" : "+v"(lsum));
+          (j < 8 ? pk0 : pk1)[j & 7] = T::pack2(te[j & 1][0], te[j & 1][1]);
+        }
+        if (nn >= 1 && nn < 17) {
+          const int j = nn - 1;
+          te[j & 1][0] = __builtin_amdgcn_exp2f(tf[j & 1][0]);
+          te[j & 1][1] = __builtin_amdgcn_exp2f(tf[j & 1][1]);
+        }
+        if (nn < 16) {
+          const floatx16& cs = nn < 8 ? c0 : c1;
+          tf[nn & 1][0] = __builtin_fmaf(cs[2 * (nn & 7)], c, -m_run);
+          tf[nn & 1][1] = __builtin_fmaf(cs[2 * (nn & 7) + 1], c, -m_run);
+        }
+      };
+      const bool copy_k = copier && s + 2 < steps, copy_v = copier && s + 1 < steps;
+      const int tile_k = (s + 2) & (NT - 1), tile_v = (s + 1) & (NT - 1);
+#pragma unroll
+      for (int r2 = 0; r2 < 16; ++r2) sn0[r2] = sn1[r2] = 0.f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        if (g & 1) sn1 = T::mfma32(f[g], qf[g >> 1], sn1);
+        else sn0 = T::mfma32(f[g], qf[g >> 1], sn0);
+        if (g < 4) {
+          if (copy_k) dma_k1(par, tile_k, g);
+        } else {
+          if (copy_v) dma_v1(par ^ 1, tile_v, g - 4);
+        }
+        f[g] = read_k(tKn, g & 1, 4 + (g >> 1));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        if (g & 1) sn1 = T::mfma32(f[g], qf[4 + (g >> 1)], sn1);
+        else sn0 = T::mfma32(f[g], qf[4 + (g >> 1)], sn0);
+        f[g] = read_vt(tV, 0, g >> 2, g & 3);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (ragged && tile_v == NT - 1) mask_tail(sn0, sn1, nv_last);
+      // the next piece's Q rows take over the registers (the scores of its first tile are computed in the next step)
+      if (r == NT - 2 && k + 1 < n) {
+        wait_vm();
+        read_q();
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int nn = 0; nn < 6; ++nn) expo_slot(nn);
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- stage B: O^T += V(s)^T P(s)^T, the rest of the softmax, the row maximum of S(s+1) ----------
+      float mxa = fmaxf(sn0[0], sn0[1]), mxb = fmaxf(sn1[0], sn1[1]);
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        u32x4 bw = {pk0[4 * cc], pk0[4 * cc + 1], pk0[4 * cc + 2], pk0[4 * cc + 3]};
+        vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const int g = cc * 4 + db;
+          o[db] = T::mfma32(f[g], bfrag, o[db]);
+          f[g] = read_vt(tV, 1, cc, db);
+          expo_slot(6 + g);
+          if (g < 4) {
+          } else if (g < 7) mxa = fmaxf(fmaxf(fmaxf(fmaxf(mxa, sn0[4 * g - 14]), sn0[4 * g - 13]), sn0[4 * g - 12]), sn0[4 * g - 11]);
+          else mxa = fmaxf(fmaxf(mxa, sn0[14]), sn0[15]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        u32x4 bw = {pk1[4 * cc], pk1[4 * cc + 1], pk1[4 * cc + 2], pk1[4 * cc + 3]};
+        vec8 bfrag = __builtin_bit_cast(vec8, bw);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const int g = cc * 4 + db;
+          o[db] = T::mfma32(f[g], bfrag, o[db]);
+          if (g < 4) expo_slot(14 + g);
+          if (g > 0) mxb = fmaxf(fmaxf(mxb, sn1[2 * g]), sn1[2 * g + 1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      l_run += lsum;
+      mx = across(fmaxf(mxa, mxb));
+
+      if (r == NT - 1) {  // the piece's last tile: the next piece starts from nothing
+        if (k >= 0 && k < n) finish_stage();
+        reset_acc();
+      }
+      if (r == 0 && k >= 1 && k <= n) finish_store(k - 1);
+    };
+
+    constexpr std::integral_constant<int, 0> even{};
+    constexpr std::integral_constant<int, 1> odd{};
+    for (int s = 0; s < steps; s += 2) {
+      step(even, s);
+      step(odd, s + 1);
+    }
+    if (phase == 1) finish_store(n - 1);  // the run ends with the last tile of wavefronts 4..7
+    __builtin_amdgcn_s_setprio(0);
+    piece0 += n;
+  }
+  wait_vm();  // no tile copy may still be on its way to LDS when the wavefront ends
 }
 
 // Folds the partial results of the pieces that attn_fwd_d128_stream_kernel computed in shares (StreamPlan):
@@ -3166,8 +3582,9 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
 //   PARAATTN_STREAM_EVEN=0|1 "stream_even"   its tail cut into shares that begin at the same keys / into equal ranges (-1 = by size)
 //   PARAATTN_SPARSE_PAIR=1   "sparse_pair"   block-sparse with 128-row query blocks: two adjacent blocks per 256-row workgroup
 //   PARAATTN_WAVE_ROWS=64    "wave_rows"     the resident-workgroup kernel as 4 wavefronts of 64 query rows instead of 8 of 32
+//   PARAATTN_SHORT_KEYS=0|1  "short_keys"    never / wherever it applies the kernel for 449..512 keys (-1 = by the number of pieces)
 struct Tuning {
-  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair, wave_rows;
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair, wave_rows, short_keys;
 };
 static Tuning& tuning() {
   static Tuning t;
@@ -3188,6 +3605,8 @@ static Tuning& tuning() {
     t.stream_even = se == 0 || se == 1 ? se : -1;
     t.sparse_pair = num("PARAATTN_SPARSE_PAIR", 0) == 1;
     t.wave_rows = num("PARAATTN_WAVE_ROWS", 0) == 64 ? 64 : 0;
+    const int sk = num("PARAATTN_SHORT_KEYS", -1);
+    t.short_keys = sk == 0 || sk == 1 ? sk : -1;
     return true;
   }();
   (void)init;
@@ -3208,6 +3627,7 @@ extern "C" int pa_set_tuning(const char* name, int value) {
   else if (!strcmp(name, "stream_even")) t.stream_even = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "sparse_pair")) t.sparse_pair = value == 1;
   else if (!strcmp(name, "wave_rows")) t.wave_rows = value == 64 ? 64 : 0;
+  else if (!strcmp(name, "short_keys")) t.short_keys = value == 0 || value == 1 ? value : -1;
   else PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: unknown knob '%s'", name);
   return PA_OK;
 }
@@ -3385,6 +3805,49 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   return true;
 }
 
+// Plan for attn_fwd_d128_short_kernel: 449..512 keys per head, head_dim 128, dense.  Worth it where a workgroup
+// gets several pieces (by default from 4 pieces per compute unit on; knob short_keys = 1: wherever it applies).
+static bool plan_short(AttnParams& p, int D) {
+  const int want = tuning().short_keys;
+  if (want == 0 || tuning().forced_bm != 0 || tuning().no_pipe) return false;
+  if (want < 0 && tuning().stream == 1) return false;  // the resident-workgroup kernel was asked for by name
+  if (D != 128 || p.causal || p.kv_len != nullptr || p.Sq <= 0) return false;
+  if (p.Skv <= (SHORT_NT - 1) * BN || p.Skv > SHORT_NT * BN) return false;
+  const int cus = device_cus();
+  if (cus <= 0) return false;
+  if ((uint64_t)(p.Skv - 1) * (uint64_t)p.ks_s * 2 + 256 >= PIPE_OOB || (uint64_t)(p.Skv - 1) * (uint64_t)p.vs_s * 2 + 256 >= PIPE_OOB ||
+      (uint64_t)(p.Sq + 255) * (uint64_t)p.qs_s * 2 + 256 >= PIPE_OOB || (uint64_t)(p.Sq + 255) * (uint64_t)p.os_s * 2 + 256 >= PIPE_OOB)
+    return false;
+  const int nqt = (p.Sq + 255) / 256;
+  const int64_t P64 = (int64_t)p.B * p.H * nqt;
+  if (P64 > 0x3fffffff) return false;
+  if (want < 0 && P64 < (int64_t)4 * cus) return false;
+  p.st.G = cus;
+  p.st.xcd_order = mi355x_layout() && (cus & 7) == 0;
+  p.st.n_pieces = (int)P64;
+  p.n_qtiles = nqt;
+  p.bm = 256;
+  p.pipe = 1;
+  p.split_s = 0;
+  return true;
+}
+
+template <typename T>
+static int launch_short(const AttnParams& p, hipStream_t stream) {
+  if (p.out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
+  const size_t smem = 4 * TILE_BYTES + 8 * 8192;  // two K and two V tiles, and 8 KB per wavefront for Q rows and outputs
+  static bool attr_done[PA_MAX_DEVICES] = {};  // benign race: the call is idempotent
+  const int dev = current_device();
+  if (dev < 0 || !attr_done[dev]) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_d128_short_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    if (dev >= 0) attr_done[dev] = true;
+  }
+  hipLaunchKernelGGL((attn_fwd_d128_short_kernel<T>), dim3((unsigned)p.st.G), dim3(512), smem, stream, p);
+  PA_CHECK_LAUNCH("attention kernel (short keys)");
+  return PA_OK;
+}
+
 template <typename T, int RB>
 static int launch_stream_rb(const AttnParams& p, hipStream_t stream) {
   const size_t smem = 4 * TILE_BYTES + 8 * 8192;  // two K and two V tiles, and a staging area for outputs
@@ -3470,6 +3933,8 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   p.causal = is_causal != 0;
   p.gate = gate;
   p.gate_want = gate_want;
+  if (!accumulate && !segs && plan_short(p, D))
+    return dtype == PA_DTYPE_BF16 ? launch_short<BF16>(p, (hipStream_t)stream) : launch_short<F16>(p, (hipStream_t)stream);
   const size_t ws_avail = workspace ? workspace_bytes : 0;
   char* ws_base = (char*)workspace;
   const int nseg = segs ? segs->n : 1;

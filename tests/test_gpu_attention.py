@@ -433,6 +433,32 @@ def test_resident_workgroup_kernel(cuda, even, bound, wave_rows, tuning):
     assert lib.pa_attn_fwd_workspace_bytes(1, 24, 4608, 4608, 128, _lib.strides3(qf), _lib.strides3(qf)) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_short_key_kernel(cuda, dtype, tuning):
+    """The kernel for 449..512 keys per head (cross-attention to a text prompt), forced on for every shape here:
+    fewer pieces than workgroups (runs of one piece), several pieces per workgroup with runs that end at a head's
+    last query tile and go on in the next head, ragged last key tiles (449, 480, 511 keys) and ragged last query
+    tiles, strided memory, several batches.  Every row against the fp64 oracle, and against the
+    resident-workgroup kernel."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    op = torch.ops.para_attn.attention_forward_with_lse
+    shapes = [(1, 2, 700, 512), (2, 3, 1380, 449), (1, 1, 31, 480), (1, 5, 256 * 3, 511),
+              (1, cus // 4 + 3, 9 * 256 - 57, 512), (2, cus // 8 + 1, 5 * 256 + 1, 500)]
+    for B, H, Sq, Skv in shapes:
+        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=Sq + Skv, dtype=dtype)
+        qd = q.to(cuda).transpose(1, 2).contiguous().transpose(1, 2)  # [B,S,H,D] memory
+        kd, vd = k.to(cuda), v.to(cuda).transpose(1, 2).contiguous().transpose(1, 2)
+        tuning("short_keys", 1)
+        out, lse = op(qd, kd, vd)
+        assert torch.equal(torch.ops.para_attn.attention_forward(qd, kd, vd), out)
+        tuning("short_keys", 0)
+        out0, lse0 = op(qd, kd, vd)
+        heads = list(range(H)) if H <= 5 else [0, 1, H // 2, H - 2, H - 1]
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, heads].float().numpy(), k[:, heads].float().numpy(), v[:, heads].float().numpy())
+        _check(out[:, heads], lse[:, heads], ref_out, ref_lse, f"short keys {(B, H, Sq, Skv, dtype)}")
+        assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
+
+
 def test_resident_workgroups_with_a_short_workspace(cuda, tuning):
     """pa_attn_fwd_lse_ws with less workspace than the plan asks for: the tail is cut into as many ranges as the
     workspace holds (still more than its pieces), or, below that, left as whole pieces; with no workspace at all the
