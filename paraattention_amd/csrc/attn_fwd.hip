@@ -2,10 +2,12 @@
 //
 // One workgroup = 4 or 8 wavefronts = 128 or 256 query rows; each wavefront owns
 // 32 query rows for the whole key sweep.  Keys/values stream through LDS in
-// tiles of 64 rows, double buffered.  Three kernels share the scheme:
+// tiles of 64 rows, double buffered.  The kernels that share the scheme:
 //   attn_fwd_kernel            any head_dim (64 when K or V spans 4 GiB or more): global -> registers -> LDS
 //   attn_fwd_d128_kernel       head_dim 128, LDS-DMA fills, 64-bit addressing
-//   attn_fwd_d128_pipe_kernel  head_dim 128, two-tile software pipeline (the default)
+//   attn_fwd_d128_pipe_kernel  head_dim 128, two-tile software pipeline
+//   attn_fwd_d128_stream_kernel  the same pipeline, resident workgroups over a list of pieces (the dense default)
+//   attn_fwd_d128_short_kernel   the same pipeline for 449..512 keys per head (cross-attention to a text prompt)
 //   attn_fwd_d64_pipe_kernel   head_dim 64, the same pipeline (the default)
 //
 // Both GEMMs run transposed so that the softmax needs no cross-lane traffic and
@@ -2873,7 +2875,6 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnP
       const int k = rel >> 3;         // its piece of the run (-1: not yet; n: no more)
       const bool copier = ((r - QI) & 7) >= 4;
       const bool was_copier = ((r - 1 - QI) & 7) >= 4;
-      floatx16 c0 = sn0, c1 = sn1;  // S(s)
 
       if (was_copier) wait_vm();  // the tile copies this wavefront issued in the step before have landed
       lds_barrier();
@@ -2884,6 +2885,28 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnP
       if (r == 1) __builtin_amdgcn_s_setprio(0);
       if (r == QI && k + 1 < n) dma_q(row_of(k + 1));
 
+      const bool copy_k = copier && s + 2 < steps, copy_v = copier && s + 1 < steps;
+      const int tile_k = (s + 2) & (NT - 1), tile_v = (s + 1) & (NT - 1);
+      if (rel < -1 || rel >= NT * n) {
+        // No piece of this wavefront is in reach (the first steps of a run for wavefronts 4..7, the last ones for
+        // 0..3): only its share of the tile copies, and what the ends of its first and last piece need.
+        if (copy_k) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dma_k1(par, tile_k, i);
+        }
+        if (copy_v) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dma_v1(par ^ 1, tile_v, i);
+        }
+        if (r == NT - 2 && k + 1 < n) {
+          wait_vm();
+          read_q();
+        }
+        if (r == 0 && k >= 1 && k <= n) finish_store(k - 1);
+        return;
+      }
+
+      floatx16 c0 = sn0, c1 = sn1;  // S(s)
 #pragma unroll
       for (int dc = 0; dc < DC; ++dc) f[dc] = read_k(tKn, dc & 1, dc >> 1);
 
@@ -2926,8 +2949,6 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnP
           tf[nn & 1][1] = __builtin_fmaf(cs[2 * (nn & 7) + 1], c, -m_run);
         }
       };
-      const bool copy_k = copier && s + 2 < steps, copy_v = copier && s + 1 < steps;
-      const int tile_k = (s + 2) & (NT - 1), tile_v = (s + 1) & (NT - 1);
 #pragma unroll
       for (int r2 = 0; r2 < 16; ++r2) sn0[r2] = sn1[r2] = 0.f;
 #pragma unroll
