@@ -23,10 +23,13 @@ def _eager(q, kb, vb, prev, cur, key_mask, block_mask):
     ratio = torch.ops.para_attn.fbcache_residual_diff(prev, cur)
     applied = torch.ops.para_attn.fbcache_apply_residual(prev, cur)
     tv = torch.ops.para_attn.taylorseer_value([cur, prev], 2, prev)
-    return [out, lse, ro, rl, uo, ul, ratio, applied, tv, mo, ml, so, wo, wl, bo, bl]
+    # 500 keys: the kernel for short key sequences (forced on by the test)
+    co, cl = torch.ops.para_attn.attention_forward_with_lse(q, kb[1][:, :, :500], vb[1][:, :, :500])
+    return [out, lse, ro, rl, uo, ul, ratio, applied, tv, mo, ml, so, wo, wl, bo, bl, co, cl]
 
 
-def test_graph_replays_match_eager(cuda):
+def test_graph_replays_match_eager(cuda, tuning):
+    tuning("short_keys", 1)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     B, H, D = 1, 4, 128
     Sq = (cus // H + 2) * 256 - 40  # a grid that takes the key-split tail and its workspace
