@@ -65,7 +65,7 @@ PA_API const char* pa_last_error(void);
  *                                           half the LDS reads per flop) instead of 8 wavefronts of 32: the same results bit for
  *                                           bit, slower as measured, kept for comparison
  *   "short_keys"   PARAATTN_SHORT_KEYS=0|1  0 / 1: never / wherever it applies the kernel for 449..512 keys per head (head_dim 128,
- *                                           dense), -1 = where a workgroup gets several query tiles
+ *                                           dense), -1 = where a workgroup gets two query tiles or more
  * Returns PA_ERR_INVALID for an unknown name or value.
  */
 PA_API int pa_set_tuning(const char* name, int value);
