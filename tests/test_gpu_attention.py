@@ -457,6 +457,10 @@ def test_short_key_kernel(cuda, dtype, tuning):
         ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, heads].float().numpy(), k[:, heads].float().numpy(), v[:, heads].float().numpy())
         _check(out[:, heads], lse[:, heads], ref_out, ref_lse, f"short keys {(B, H, Sq, Skv, dtype)}")
         assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
+        tuning("short_keys", -1)  # by itself the planner takes it from two query tiles per compute unit on
+        out_d, lse_d = op(qd, kd, vd)
+        want = (out, lse) if B * H * ((Sq + 255) // 256) >= 2 * cus else (out0, lse0)
+        assert torch.equal(out_d, want[0]) and torch.equal(lse_d, want[1]), (B, H, Sq, Skv)
 
 
 def test_resident_workgroups_with_a_short_workspace(cuda, tuning):
