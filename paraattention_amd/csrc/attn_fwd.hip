@@ -2623,7 +2623,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
 // Dense, not causal, no per-batch key counts, no accumulation.
 // ---------------------------------------------------------------------------------------------
 constexpr int SHORT_NT = 8;  // key tiles of a piece
-constexpr int SHORT_QI = 5;  // step of a piece (0..7) at whose start the next piece's Q rows are sent for
+constexpr int SHORT_QI = 5;  // step of a piece (0..7) in which the next piece's Q rows are sent for
 
 template <typename T>
 __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnParams p) {
@@ -2883,7 +2883,6 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnP
       // it is given that lead.
       if (r == QI) __builtin_amdgcn_s_setprio(2);
       if (r == 1) __builtin_amdgcn_s_setprio(0);
-      if (r == QI && k + 1 < n) dma_q(row_of(k + 1));
 
       const bool copy_k = copier && s + 2 < steps, copy_v = copier && s + 1 < steps;
       const int tile_k = (s + 2) & (NT - 1), tile_v = (s + 1) & (NT - 1);
@@ -2898,6 +2897,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnP
 #pragma unroll
           for (int i = 0; i < 4; ++i) dma_v1(par ^ 1, tile_v, i);
         }
+        if (r == QI && k + 1 < n) dma_q(row_of(k + 1));
         if (r == NT - 2 && k + 1 < n) {
           wait_vm();
           read_q();
@@ -2970,6 +2970,9 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnP
         f[g] = read_vt(tV, 0, g >> 2, g & 3);
         __builtin_amdgcn_sched_barrier(0);
       }
+      // the next piece's Q rows are sent for here, between the two GEMMs, and not at the top of the step, where the
+      // eight copy instructions would stand in front of the first fragment reads (measured: 2.2 % of the launch)
+      if (r == QI && k + 1 < n) dma_q(row_of(k + 1));
       if (ragged && tile_v == NT - 1) mask_tail(sn0, sn1, nv_last);
       // the next piece's Q rows take over the registers (the scores of its first tile are computed in the next step)
       if (r == NT - 2 && k + 1 < n) {
