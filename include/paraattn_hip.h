@@ -64,6 +64,8 @@ PA_API const char* pa_last_error(void);
  *   "wave_rows"    PARAATTN_WAVE_ROWS=64    64: the kernel with resident workgroups runs as 4 wavefronts of 64 query rows (one per SIMD,
  *                                           half the LDS reads per flop) instead of 8 wavefronts of 32: the same results bit for
  *                                           bit, slower as measured, kept for comparison
+ *   "sparse_order" PARAATTN_SPARSE_ORDER=0  0: block-sparse launches take the query blocks of a head in their own order instead of
+ *                                           longest list of key ranges first (1, the default)
  *   "short_keys"   PARAATTN_SHORT_KEYS=0|1  0 / 1: never / wherever it applies the kernel for 449..512 keys per head (head_dim 128,
  *                                           dense), -1 = where a workgroup gets two query tiles or more
  * Returns PA_ERR_INVALID for an unknown name or value.
@@ -263,7 +265,8 @@ PA_API size_t pa_attn_fwd_call_workspace_bytes(int B, int H, int Sq, int Skv, in
  * runs_ws: int32 workspace of at least pa_blocksparse_workspace_bytes() bytes;
  * it receives, per (hm, query segment), the list of key ranges the kernel
  * walks (the mask's runs of kept blocks, merged, exactly as
- * sparse_attn.py:215-234 scans them).
+ * sparse_attn.py:215-234 scans them), and behind the lists the order in which
+ * the query blocks of a head are started (longest list first; up to 2048 blocks).
  * A query block that keeps no key at all yields out = 0 and lse = -inf.
  */
 PA_API int pa_attn_fwd_blocksparse(const void* q, const void* k, const void* v, void* out, float* lse,

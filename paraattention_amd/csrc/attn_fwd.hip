@@ -86,6 +86,7 @@ struct AttnParams {
   int causal;             // dense: query row i sees keys 0..i only (torch's is_causal, top-left aligned)
   // block-sparse only
   const int32_t* runs;  // count[Hm*nSeg] then range[Hm*nSeg][cap][2]
+  const int32_t* order;  // optional [Hm][nQ]: the query blocks of a head by falling number of key tiles (launch order)
   int Hm, nQ, cap;
   int q_lo, q_block;
   int pair;  // block-sparse: each 256-row workgroup holds two 128-row query blocks and walks the union of their ranges
@@ -216,8 +217,11 @@ __device__ __forceinline__ void decode_block(const AttnParams& p, int qt, int he
       int r = qt - p.tiles_left;
       int blk = r / p.tiles_per_block;
       if (blk < p.nQ) {
-        seg = 1 + blk;
         tin = r - blk * p.tiles_per_block;
+        // workgroups are started in the order of their numbers: the longest lists of a head first, so that the
+        // launch does not end on a few long ones
+        if (p.order != nullptr) blk = p.order[(p.Hm == 1 ? 0 : head) * p.nQ + blk];
+        seg = 1 + blk;
         row_begin = p.q_lo + blk * p.q_block + tin * p.bm;
         row_end = p.q_lo + (blk + 1) * p.q_block;
       } else {
@@ -3309,6 +3313,34 @@ __global__ __launch_bounds__(64) void build_pair_runs_kernel(const uint8_t* mask
 constexpr int BOUND_G = 1024;                                   // blocks per tensor
 constexpr size_t BOUND_WS_BYTES = (2 * BOUND_G + 64) * 4;       // partial maxima + the flag word (+ padding)
 // with the keys in n segments: one set of partial maxima per segment, then the flag word
+// The query blocks of every head by falling number of key tiles (ties by block number): the launch order of the
+// block-sparse kernels.  Workgroups start in the order of their numbers as slots fall free, so a launch that hands
+// the lists out as they come ends on whatever long lists happen to come late (4 % of the launch on a mask whose
+// lists differ by 9 % rms); longest first within a head, it ends on the short ones.  One workgroup per mask head.
+constexpr int SPARSE_ORDER_MAX_BLOCKS = 2048;  // the ranking below is quadratic in the blocks of a head
+__global__ __launch_bounds__(256) void sparse_order_kernel(const int32_t* runs, int Hm, int nQ, int cap, int32_t* order) {
+  extern __shared__ int len_of[];
+  const int hm = blockIdx.x, nseg = nQ + 2;
+  for (int blk = threadIdx.x; blk < nQ; blk += 256) {
+    const int sidx = hm * nseg + 1 + blk;
+    const int cnt = runs[sidx];
+    const int32_t* r = runs + (size_t)Hm * nseg + (size_t)sidx * cap * 2;
+    int tiles = 0;
+    for (int i = 0; i < cnt; ++i) tiles += (r[2 * i + 1] - r[2 * i] + BN - 1) / BN;
+    len_of[blk] = tiles;
+  }
+  __syncthreads();
+  for (int blk = threadIdx.x; blk < nQ; blk += 256) {
+    const int mine = len_of[blk];
+    int rank = 0;
+    for (int j = 0; j < nQ; ++j) {
+      const int other = len_of[j];
+      rank += (other > mine || (other == mine && j < blk)) ? 1 : 0;
+    }
+    order[(size_t)hm * nQ + rank] = blk;
+  }
+}
+
 static inline size_t bound_ws_bytes(int nseg) { return ((size_t)2 * BOUND_G * (nseg < 1 ? 1 : nseg) + 64) * 4; }
 
 template <typename T, int D>
@@ -3451,6 +3483,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.scale_log2 = scale * LOG2E;
   p.kv_len = nullptr;
   p.runs = nullptr;
+  p.order = nullptr;
   p.Hm = 0; p.nQ = 0; p.cap = 0; p.q_lo = 0; p.q_block = 0; p.pair = 0; p.tiles_left = 0; p.tiles_per_block = 0;
   p.bm = BM; p.pipe = 0;
   p.xcd_chunk = 0;
@@ -3606,9 +3639,10 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
 //   PARAATTN_STREAM_EVEN=0|1 "stream_even"   its tail cut into shares that begin at the same keys / into equal ranges (-1 = by size)
 //   PARAATTN_SPARSE_PAIR=1   "sparse_pair"   block-sparse with 128-row query blocks: two adjacent blocks per 256-row workgroup
 //   PARAATTN_WAVE_ROWS=64    "wave_rows"     the resident-workgroup kernel as 4 wavefronts of 64 query rows instead of 8 of 32
+//   PARAATTN_SPARSE_ORDER=0  "sparse_order"  block-sparse: 0 = the query blocks of a head in their own order instead of longest list first
 //   PARAATTN_SHORT_KEYS=0|1  "short_keys"    never / wherever it applies the kernel for 449..512 keys (-1 = by the number of pieces)
 struct Tuning {
-  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair, wave_rows, short_keys;
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair, wave_rows, short_keys, sparse_order;
 };
 static Tuning& tuning() {
   static Tuning t;
@@ -3631,6 +3665,7 @@ static Tuning& tuning() {
     t.wave_rows = num("PARAATTN_WAVE_ROWS", 0) == 64 ? 64 : 0;
     const int sk = num("PARAATTN_SHORT_KEYS", -1);
     t.short_keys = sk == 0 || sk == 1 ? sk : -1;
+    t.sparse_order = num("PARAATTN_SPARSE_ORDER", 1) != 0;
     return true;
   }();
   (void)init;
@@ -3652,6 +3687,7 @@ extern "C" int pa_set_tuning(const char* name, int value) {
   else if (!strcmp(name, "sparse_pair")) t.sparse_pair = value == 1;
   else if (!strcmp(name, "wave_rows")) t.wave_rows = value == 64 ? 64 : 0;
   else if (!strcmp(name, "short_keys")) t.short_keys = value == 0 || value == 1 ? value : -1;
+  else if (!strcmp(name, "sparse_order")) t.sparse_order = value != 0;
   else PA_FAIL(PA_ERR_INVALID, "pa_set_tuning: unknown knob '%s'", name);
   return PA_OK;
 }
@@ -4259,9 +4295,16 @@ extern "C" size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK) {
   if (Hm <= 0 || nQ <= 0 || nK <= 0) return 0;
   const size_t nseg = (size_t)nQ + 2;
   const size_t cap = (size_t)nK / 2 + 3;
-  const size_t single = sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2);
+  const size_t single = sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2 + (size_t)Hm * nQ);  // the lists, then the launch order
   const size_t pairs = pair_runs_bytes(Hm, nQ, nK);
   return single > pairs ? single : pairs;
+}
+
+// Where the launch order of the query blocks lies in a buffer of single-block lists (words from its start).
+static size_t order_offset_words(int Hm, int nQ, int nK) {
+  const size_t nseg = (size_t)nQ + 2;
+  const size_t cap = (size_t)nK / 2 + 3;
+  return (size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2;
 }
 
 extern "C" int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int nQ, int nK, int Skv,
@@ -4279,6 +4322,11 @@ extern "C" int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int 
   hipLaunchKernelGGL(build_runs_kernel, dim3(total), dim3(64), 0, (hipStream_t)stream,
                      block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, cap, runs_ws);
   PA_CHECK_LAUNCH("build_runs_kernel");
+  if (nQ <= SPARSE_ORDER_MAX_BLOCKS) {
+    hipLaunchKernelGGL(sparse_order_kernel, dim3(Hm), dim3(256), (size_t)nQ * sizeof(int), (hipStream_t)stream,
+                       (const int32_t*)runs_ws, Hm, nQ, cap, runs_ws + order_offset_words(Hm, nQ, nK));
+    PA_CHECK_LAUNCH("sparse_order_kernel");
+  }
   return PA_OK;
 }
 
@@ -4293,6 +4341,7 @@ static int blocksparse_launch(const void* q, const void* k, const void* v, void*
   p.runs = runs;
   p.Hm = Hm; p.nQ = nQ; p.cap = nK / 2 + 3;
   p.q_lo = q_lo; p.q_block = q_block;
+  if (!pair && nQ <= SPARSE_ORDER_MAX_BLOCKS && tuning().sparse_order) p.order = runs + order_offset_words(Hm, nQ, nK);
   choose_kernel(p, D, (q_block % 256 == 0 && q_lo % 256 == 0) ? 256 : 128, false, 0, nullptr);
   if (pair) {  // `runs` holds the lists of pairs: 256-row workgroups over nQ / 2 double blocks
     if (!p.pipe || D != 128 || q_block != 128 || nQ % 2 != 0 || q_lo % 256 != 0)

@@ -690,6 +690,21 @@ def block_sparse_runs(block_mask, Skv, kv_lo=0, kv_hi=-1):
     return count, ranges
 
 
+def block_sparse_launch_order(block_mask, Skv, kv_lo=0, kv_hi=-1):
+    """[Hm, nQ] int32: the query blocks of each mask head in the order a launch starts them (the longest list of
+    64-key tiles first, ties by block number), as the device built it; None beyond 2048 blocks per head, where the
+    launch keeps the blocks' own order."""
+    if block_mask.ndim == 2:
+        block_mask = block_mask.unsqueeze(0)
+    Hm, nQ, nK = block_mask.shape
+    if nQ > 2048:
+        return None
+    ws = block_sparse_key_runs(block_mask, Skv, kv_lo, kv_hi)
+    nseg, cap = nQ + 2, nK // 2 + 3
+    first = Hm * nseg + Hm * nseg * cap * 2
+    return ws[first : first + Hm * nQ].view(Hm, nQ)
+
+
 # ---------------------------------------------------------------------------------
 # First Block Cache reductions
 # ---------------------------------------------------------------------------------

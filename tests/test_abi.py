@@ -81,7 +81,7 @@ def test_argument_validation_without_device_work():
     assert lib.pa_merge_lse(a, 2, a, a, 0, a, a, 2, a, 4, 12, None) == _lib.PA_ERR_UNSUPPORTED
     assert lib.pa_merge_lse(a, 2, a, a, 0, a, a, 0, a, 4, 16, None) == _lib.PA_ERR_INVALID
     # block-sparse geometry
-    assert lib.pa_blocksparse_workspace_bytes(24, 256, 256) == 4 * (24 * 258 + 24 * 258 * 131 * 2)
+    assert lib.pa_blocksparse_workspace_bytes(24, 256, 256) == 4 * (24 * 258 + 24 * 258 * 131 * 2 + 24 * 256)  # counts, ranges, launch order
     assert lib.pa_blocksparse_workspace_bytes(0, 1, 1) == 0
     assert lib.pa_blocksparse_build_runs(a, 1, 2, 3, 100, 0, 64, a, 4096, None) == _lib.PA_ERR_INVALID  # 3*64 > 100
     assert lib.pa_blocksparse_build_runs(a, 1, 2, 3, 192, 0, 64, a, 8, None) == _lib.PA_ERR_WORKSPACE
@@ -101,12 +101,12 @@ def test_tuning_knobs_are_validated():
         assert lib.pa_set_tuning(b"bm", 100) == _lib.PA_ERR_INVALID and b"bm" in lib.pa_last_error()
         assert lib.pa_set_tuning(b"no_such_knob", 1) == _lib.PA_ERR_INVALID
         assert lib.pa_set_tuning(None, 1) == _lib.PA_ERR_INVALID
-        for name in (b"no_pipe", b"no_split", b"no_xcd_order", b"bound", b"stream", b"stream_even", b"sparse_pair", b"wave_rows", b"short_keys"):
+        for name in (b"no_pipe", b"no_split", b"no_xcd_order", b"bound", b"stream", b"stream_even", b"sparse_pair", b"wave_rows", b"short_keys", b"sparse_order"):
             assert lib.pa_set_tuning(name, 1) == _lib.PA_OK
         with pytest.raises(ValueError):
             _lib.set_tuning("bm", 64)
     finally:
-        for name, val in (("no_pipe", 0), ("bm", 0), ("no_split", 0), ("no_xcd_order", 0), ("bound", -1), ("stream", -1), ("stream_even", -1), ("sparse_pair", 0), ("wave_rows", 0), ("short_keys", -1)):
+        for name, val in (("no_pipe", 0), ("bm", 0), ("no_split", 0), ("no_xcd_order", 0), ("bound", -1), ("stream", -1), ("stream_even", -1), ("sparse_pair", 0), ("wave_rows", 0), ("short_keys", -1), ("sparse_order", 1)):
             _lib.set_tuning(name, val)
 
 

@@ -44,6 +44,40 @@ def test_runs_reproduce_mask_bit_exact(cuda, Hm, nQ, nK):
     assert (count[:, 0] == 1).all() and (count[:, -1] == 1).all()
 
 
+@pytest.mark.parametrize("Hm,nQ,nK,kb", [(1, 1, 1, 128), (2, 9, 7, 100), (3, 40, 33, 16), (24, 256, 256, 128)])
+def test_launch_order_is_longest_list_first(cuda, Hm, nQ, nK, kb):
+    mask, _ = inputs.block_mask(Hm, nQ, nK, seed=nQ)
+    Skv = nK * kb + 40
+    count, ranges = ops.block_sparse_runs(mask.to(cuda), Skv=Skv, kv_lo=24, kv_hi=24 + nK * kb)
+    order = ops.block_sparse_launch_order(mask.to(cuda), Skv=Skv, kv_lo=24, kv_hi=24 + nK * kb).cpu().numpy()
+    count, ranges = count.cpu().numpy(), ranges.cpu().numpy()
+    for h in range(Hm):
+        tiles = np.array([sum(-(-(int(ranges[h, i + 1, r, 1]) - int(ranges[h, i + 1, r, 0])) // 64) for r in range(count[h, i + 1])) for i in range(nQ)])
+        want = np.argsort(-tiles, kind="stable")  # falling number of 64-key tiles, ties by block number
+        assert np.array_equal(order[h], want), h
+
+
+def test_launch_order_leaves_results_alone(cuda, tuning):
+    """Which query block a workgroup takes (knob "sparse_order") changes when a block is computed, not what: the
+    same bits either way, with margins, several tiles per block, per-head masks and both head dims."""
+    op = torch.ops.para_attn.attention_forward_block_sparse
+    rng = np.random.default_rng(11)
+    for case, (H, nQ, nK, qb, kb, q_lo, q_tail, kv_lo, kv_tail, D, per_head) in enumerate([
+        (3, 12, 10, 128, 128, 0, 0, 0, 0, 128, True), (2, 5, 9, 256, 64, 256, 37, 24, 12, 128, True),
+        (2, 7, 6, 128, 100, 128, 50, 8, 0, 64, False), (1, 20, 16, 64, 32, 0, 0, 0, 64, 128, True),
+    ]):
+        Sq, Skv = q_lo + nQ * qb + q_tail, kv_lo + nK * kb + kv_tail
+        bm = torch.from_numpy(rng.random((H if per_head else 1, nQ, nK)) < rng.uniform(0.1, 0.9, size=(1, nQ, 1)))
+        bm2 = bm if per_head else bm[0]
+        q, k, v = (t.to(cuda) for t in inputs.qkv(1, H, Sq, Skv, D, seed=700 + case))
+        args = (q, k, v, bm2.to(cuda), q_lo, q_lo + nQ * qb, kv_lo, kv_lo + nK * kb)
+        tuning("sparse_order", 0)
+        out0, lse0 = op(*args)
+        tuning("sparse_order", 1)
+        out1, lse1 = op(*args)
+        assert torch.equal(out0, out1) and torch.equal(lse0, lse1), case
+
+
 def test_runs_word_boundaries(cuda):
     # rows that exercise the 64-block voting words: kept block at bit 63, runs crossing words, all kept, none kept
     nK = 200
