@@ -266,7 +266,8 @@ PA_API size_t pa_attn_fwd_call_workspace_bytes(int B, int H, int Sq, int Skv, in
  * it receives, per (hm, query segment), the list of key ranges the kernel
  * walks (the mask's runs of kept blocks, merged, exactly as
  * sparse_attn.py:215-234 scans them), and behind the lists the order in which
- * the query blocks of a head are started (longest list first; up to 2048 blocks).
+ * the query blocks of a head are started (the block that keeps most key blocks
+ * first; up to 2048 blocks).
  * A query block that keeps no key at all yields out = 0 and lse = -inf.
  */
 PA_API int pa_attn_fwd_blocksparse(const void* q, const void* k, const void* v, void* out, float* lse,

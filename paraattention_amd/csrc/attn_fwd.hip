@@ -3169,7 +3169,7 @@ __global__ __launch_bounds__(256) void attn_split_merge_kernel(const AttnParams 
 // Segments 0 and nQ+1 are the dense query margins.
 __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int Hm, int nQ, int nK,
                                                         int Skv, int kv_lo, int kv_block, int cap,
-                                                        int32_t* ws) {
+                                                        int32_t* ws, int32_t* kept_out) {
   const int nseg = nQ + 2;
   const int idx = blockIdx.x;  // grid = Hm * nseg
   const int lane = threadIdx.x;
@@ -3197,10 +3197,12 @@ __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int
   const bool first_kept = row[0] != 0, last_kept = row[nK - 1] != 0;
   const int first_idx = left && !first_kept ? 1 : 0;  // range index of the first run
   int begins = 0, ends = 0;                           // runs begun / ended in the passes so far
+  int kept = 0;                                       // kept key blocks of this query block
   const uint64_t below = lane == 0 ? 0 : (~0ull >> (64 - lane));
   for (int base = 0; base < nK; base += 64) {
     const int j = base + lane;
     const bool keep = j < nK && row[j] != 0;
+    kept += __builtin_popcountll(__ballot(keep));
     const bool begin = keep && (j == 0 || row[j - 1] == 0);
     const bool end = keep && (j == nK - 1 || row[j + 1] == 0);
     const uint64_t bb = __ballot(begin), eb = __ballot(end);
@@ -3227,6 +3229,7 @@ __global__ __launch_bounds__(64) void build_runs_kernel(const uint8_t* mask, int
       ++n;
     }
     *cnt = n;
+    if (kept_out != nullptr) kept_out[(size_t)hm * nQ + (seg - 1)] = kept;  // what sparse_order_kernel ranks the block by
   }
 }
 
@@ -3313,22 +3316,18 @@ __global__ __launch_bounds__(64) void build_pair_runs_kernel(const uint8_t* mask
 constexpr int BOUND_G = 1024;                                   // blocks per tensor
 constexpr size_t BOUND_WS_BYTES = (2 * BOUND_G + 64) * 4;       // partial maxima + the flag word (+ padding)
 // with the keys in n segments: one set of partial maxima per segment, then the flag word
-// The query blocks of every head by falling number of key tiles (ties by block number): the launch order of the
-// block-sparse kernels.  Workgroups start in the order of their numbers as slots fall free, so a launch that hands
-// the lists out as they come ends on whatever long lists happen to come late (4 % of the launch on a mask whose
-// lists differ by 9 % rms); longest first within a head, it ends on the short ones.  One workgroup per mask head.
+// The query blocks of every head by falling number of kept key blocks (ties by block number): the launch order of
+// the block-sparse kernels.  Workgroups start in the order of their numbers as slots fall free, so a launch that
+// hands the lists out as they come ends on whatever long lists happen to come late (4 % of the launch on a mask
+// whose lists differ by 9 % rms), and workgroups that run side by side are at different places of the key axis.
+// Longest first within a head, the launch ends on the short lists, and neighbours in the order are lists of
+// nearly the same length, which start and end together and sweep the keys in step: half the reads from beyond
+// the L2 on the same mask.  One workgroup per mask head; `kept` comes from build_runs_kernel.
 constexpr int SPARSE_ORDER_MAX_BLOCKS = 2048;  // the ranking below is quadratic in the blocks of a head
-__global__ __launch_bounds__(256) void sparse_order_kernel(const int32_t* runs, int Hm, int nQ, int cap, int32_t* order) {
+__global__ __launch_bounds__(256) void sparse_order_kernel(const int32_t* kept, int nQ, int32_t* order) {
   extern __shared__ int len_of[];
-  const int hm = blockIdx.x, nseg = nQ + 2;
-  for (int blk = threadIdx.x; blk < nQ; blk += 256) {
-    const int sidx = hm * nseg + 1 + blk;
-    const int cnt = runs[sidx];
-    const int32_t* r = runs + (size_t)Hm * nseg + (size_t)sidx * cap * 2;
-    int tiles = 0;
-    for (int i = 0; i < cnt; ++i) tiles += (r[2 * i + 1] - r[2 * i] + BN - 1) / BN;
-    len_of[blk] = tiles;
-  }
+  const int hm = blockIdx.x;
+  for (int blk = threadIdx.x; blk < nQ; blk += 256) len_of[blk] = kept[(size_t)hm * nQ + blk];
   __syncthreads();
   for (int blk = threadIdx.x; blk < nQ; blk += 256) {
     const int mine = len_of[blk];
@@ -4295,7 +4294,7 @@ extern "C" size_t pa_blocksparse_workspace_bytes(int Hm, int nQ, int nK) {
   if (Hm <= 0 || nQ <= 0 || nK <= 0) return 0;
   const size_t nseg = (size_t)nQ + 2;
   const size_t cap = (size_t)nK / 2 + 3;
-  const size_t single = sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2 + (size_t)Hm * nQ);  // the lists, then the launch order
+  const size_t single = sizeof(int32_t) * ((size_t)Hm * nseg + (size_t)Hm * nseg * cap * 2 + (size_t)2 * Hm * nQ);  // the lists, the launch order, the kept blocks per list
   const size_t pairs = pair_runs_bytes(Hm, nQ, nK);
   return single > pairs ? single : pairs;
 }
@@ -4319,12 +4318,15 @@ extern "C" int pa_blocksparse_build_runs(const uint8_t* block_mask, int Hm, int 
     PA_FAIL(PA_ERR_WORKSPACE, "runs workspace too small");
   const int total = Hm * (nQ + 2);
   const int cap = nK / 2 + 3;
+  int32_t* const order = runs_ws + order_offset_words(Hm, nQ, nK);
+  int32_t* const kept = order + (size_t)Hm * nQ;
+  const bool ranked = nQ <= SPARSE_ORDER_MAX_BLOCKS;
   hipLaunchKernelGGL(build_runs_kernel, dim3(total), dim3(64), 0, (hipStream_t)stream,
-                     block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, cap, runs_ws);
+                     block_mask, Hm, nQ, nK, Skv, kv_lo, kv_block, cap, runs_ws, ranked ? kept : nullptr);
   PA_CHECK_LAUNCH("build_runs_kernel");
-  if (nQ <= SPARSE_ORDER_MAX_BLOCKS) {
+  if (ranked) {
     hipLaunchKernelGGL(sparse_order_kernel, dim3(Hm), dim3(256), (size_t)nQ * sizeof(int), (hipStream_t)stream,
-                       (const int32_t*)runs_ws, Hm, nQ, cap, runs_ws + order_offset_words(Hm, nQ, nK));
+                       (const int32_t*)kept, nQ, order);
     PA_CHECK_LAUNCH("sparse_order_kernel");
   }
   return PA_OK;

@@ -691,8 +691,8 @@ def block_sparse_runs(block_mask, Skv, kv_lo=0, kv_hi=-1):
 
 
 def block_sparse_launch_order(block_mask, Skv, kv_lo=0, kv_hi=-1):
-    """[Hm, nQ] int32: the query blocks of each mask head in the order a launch starts them (the longest list of
-    64-key tiles first, ties by block number), as the device built it; None beyond 2048 blocks per head, where the
+    """[Hm, nQ] int32: the query blocks of each mask head in the order a launch starts them (the block that keeps most
+    key blocks first, ties by block number), as the device built it; None beyond 2048 blocks per head, where the
     launch keeps the blocks' own order."""
     if block_mask.ndim == 2:
         block_mask = block_mask.unsqueeze(0)

@@ -81,7 +81,7 @@ def test_argument_validation_without_device_work():
     assert lib.pa_merge_lse(a, 2, a, a, 0, a, a, 2, a, 4, 12, None) == _lib.PA_ERR_UNSUPPORTED
     assert lib.pa_merge_lse(a, 2, a, a, 0, a, a, 0, a, 4, 16, None) == _lib.PA_ERR_INVALID
     # block-sparse geometry
-    assert lib.pa_blocksparse_workspace_bytes(24, 256, 256) == 4 * (24 * 258 + 24 * 258 * 131 * 2 + 24 * 256)  # counts, ranges, launch order
+    assert lib.pa_blocksparse_workspace_bytes(24, 256, 256) == 4 * (24 * 258 + 24 * 258 * 131 * 2 + 2 * 24 * 256)  # counts, ranges, launch order, kept blocks per list
     assert lib.pa_blocksparse_workspace_bytes(0, 1, 1) == 0
     assert lib.pa_blocksparse_build_runs(a, 1, 2, 3, 100, 0, 64, a, 4096, None) == _lib.PA_ERR_INVALID  # 3*64 > 100
     assert lib.pa_blocksparse_build_runs(a, 1, 2, 3, 192, 0, 64, a, 8, None) == _lib.PA_ERR_WORKSPACE

@@ -48,12 +48,9 @@ def test_runs_reproduce_mask_bit_exact(cuda, Hm, nQ, nK):
 def test_launch_order_is_longest_list_first(cuda, Hm, nQ, nK, kb):
     mask, _ = inputs.block_mask(Hm, nQ, nK, seed=nQ)
     Skv = nK * kb + 40
-    count, ranges = ops.block_sparse_runs(mask.to(cuda), Skv=Skv, kv_lo=24, kv_hi=24 + nK * kb)
     order = ops.block_sparse_launch_order(mask.to(cuda), Skv=Skv, kv_lo=24, kv_hi=24 + nK * kb).cpu().numpy()
-    count, ranges = count.cpu().numpy(), ranges.cpu().numpy()
     for h in range(Hm):
-        tiles = np.array([sum(-(-(int(ranges[h, i + 1, r, 1]) - int(ranges[h, i + 1, r, 0])) // 64) for r in range(count[h, i + 1])) for i in range(nQ)])
-        want = np.argsort(-tiles, kind="stable")  # falling number of 64-key tiles, ties by block number
+        want = np.argsort(-mask[h].sum(-1).numpy(), kind="stable")  # falling number of kept key blocks, ties by block number
         assert np.array_equal(order[h], want), h
 
 
