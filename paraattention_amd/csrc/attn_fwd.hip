@@ -2621,7 +2621,8 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
 // matrix cores busy.  The half that is in mid-piece also issues all the tile copies; the half that changes
 // pieces issues none for four steps and therefore never waits at a barrier for its own loads and stores (one
 // counter covers tile copies, Q loads and output stores): its next Q rows travel into the wavefront's own 8 KB
-// of LDS a step and a half before they are needed, and its output leaves through the same 8 KB.
+// of LDS a step before they are needed, and its output leaves through the same 8 KB in two parts, each behind
+// the last MFMA of a step.  The wavefront that changes pieces has priority over the other one of its SIMD.
 // Workgroup g takes the pieces [g P / G, (g + 1) P / G); consecutive pieces of one head form a run of
 // 8 n + 4 steps (wavefronts 4..7 idle for the first four, 0..3 for the last four).
 // Dense, not causal, no per-batch key counts, no accumulation.
