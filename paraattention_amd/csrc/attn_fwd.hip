@@ -3744,6 +3744,10 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
   // +4..10 % from 4608 keys up, -4 % at 512 keys
   const double gain256 = !mi355x_layout() ? 1.0 : kv_tiles >= 32 ? 1.055 : 0.95;
   bool use256 = cus > 0 && n256 >= cus && r256 / gain256 < r128;
+  // is_causal: workgroups differ in length and are started longest first, so whole rounds mean nothing; measured
+  // (B1, 24..40 heads): 128 rows are 3..12 % faster from 2048 to 32768 keys (the finer grain fills the chip's
+  // tail), 256 rows 8 % faster at 119056 (half the tile copies per flop, a third of the reads from beyond the L2)
+  if (p.causal) use256 = cus > 0 && n256 >= cus && kv_tiles >= 1024;
   if (forced == 128) use256 = false;
   if (forced == 256) use256 = true;
   const SplitPlan& pl = use256 ? p256 : p128;
