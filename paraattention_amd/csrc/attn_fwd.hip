@@ -3722,7 +3722,11 @@ static void choose_kernel(AttnParams& p, int D, int q_block, bool dense, size_t 
     return finish();
   }
   if (!dense) {  // block-sparse: workgroups differ in length, no split
-    if (forced == 256 && q_block % 256 == 0) p.bm = 256;
+    // query blocks that are multiples of 256 rows take 256-row workgroups where there are two or more of them per
+    // compute unit (measured on a 30 % mask of 256 x 256 blocks, B1 H24 S32768: 3.46 against 3.54 ms)
+    const int cus = device_cus();
+    const bool enough = cus > 0 && (int64_t)p.B * p.H * ((p.Sq + 255) / 256) >= (int64_t)2 * cus;
+    if (q_block % 256 == 0 && (forced == 256 || (forced == 0 && enough))) p.bm = 256;
     return finish();
   }
   const int cus = device_cus();
