@@ -3814,6 +3814,10 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   const int64_t P64 = (int64_t)p.B * p.H * nqt;
   if (L64 > 0x3fffffff || P64 > 0x3fffffff) return false;
   const int L = (int)L64, P = (int)P64;
+  // Small problems -- fewer pieces than compute units and no more than 6144 key-tile steps in all -- are left to the
+  // kernels with one workgroup per query tile: this kernel would cut every piece into ranges and pay a second
+  // launch to fold them, which at 30..80 us per call is 8..40 % (measured over 2..64 heads and 576..4608 tokens).
+  if (want < 0 && !multi && P < cus && (int64_t)P * L <= 6144) return false;
   // Taken wherever it applies (measured against attn_fwd_d128_pipe_kernel + key-split tail on one box: 119056 keys
   // +0.6 %, Wan self-attention +0.9 %, a ring sweep's block +3.5 %, the sweep in one launch +1.3 %, 16k / 8k / 6k /
   // 3k tokens +1.5 / +2.4 / +7 / +7 %, FLUX +10..17 %, cross-attention to 512 keys +6 %): the hot loop is the same,
