@@ -74,6 +74,7 @@ def test_noalloc_with_resident_workgroups(cuda, tuning):
     results lie in the scratch): bit for bit the workspace entry's result, on two calls in a row."""
     lib = _lib.load()
     tuning("bound", 1)
+    tuning("stream", 1)  # the second, small problem would by itself go to the kernels with one workgroup per query tile
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     B, D = 1, 128
     for H, Sq, Skv in ((4, (cus // 4 + 25) * 256 - 50, 64 * 30 + 11), (3, 9 * 256 + 3, 64 * 9)):
