@@ -463,6 +463,24 @@ def test_short_key_kernel(cuda, dtype, tuning):
         assert torch.equal(out_d, want[0]) and torch.equal(lse_d, want[1]), (B, H, Sq, Skv)
 
 
+@pytest.mark.parametrize("scale", [1.0, 0.3])
+def test_short_key_kernel_large_logits(cuda, scale, tuning):
+    """Logits of a few hundred through the kernel for short key sequences: the running maximum rises from tile to
+    tile (keys sorted by their projection on a fixed direction, ascending, so that later tiles hold the larger
+    scores; both halves of the workgroup, which walk the tiles in different orders), against the fp64 oracle."""
+    tuning("short_keys", 1)
+    B, H, Sq, Skv = 1, 3, 700, 507
+    q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=11)
+    q = q * 3
+    d = torch.randn(128, generator=torch.Generator().manual_seed(1))
+    order = torch.argsort((k.float() @ d), dim=2)
+    k = torch.gather(k, 2, order[..., None].expand_as(k))
+    q = (q.float() + 2.0 * d).bfloat16()
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale)
+    out, lse = torch.ops.para_attn.attention_forward_with_lse(q.to(cuda), k.to(cuda), v.to(cuda), scale=scale)
+    _check(out, lse, ref_out, ref_lse, f"short keys, large logits, scale {scale}")
+
+
 def test_resident_workgroups_with_a_short_workspace(cuda, tuning):
     """pa_attn_fwd_lse_ws with less workspace than the plan asks for: the tail is cut into as many ranges as the
     workspace holds (still more than its pieces), or, below that, left as whole pieces; with no workspace at all the
