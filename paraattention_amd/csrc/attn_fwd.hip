@@ -3344,11 +3344,13 @@ __global__ __launch_bounds__(256) void sparse_order_kernel(const int32_t* kept, 
 static inline size_t bound_ws_bytes(int nseg) { return ((size_t)2 * BOUND_G * (nseg < 1 ? 1 : nseg) + 64) * 4; }
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnParams p, float* part, const void* keys, int n_keys) {
+__global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnParams p, float* part, const void* keys, int n_keys, int q_too) {
   constexpr int LPR = D / 8;       // lanes per row: 8 elements each
   constexpr int RPB = 256 / LPR;   // rows per block and step
-  const bool is_k = blockIdx.x >= BOUND_G;
-  const int blk = is_k ? blockIdx.x - BOUND_G : blockIdx.x;
+  // q_too: BOUND_G blocks for Q, then BOUND_G for the keys; otherwise the key blocks alone (a further key segment of
+  // a sweep: the Q rows were looked at with the first)
+  const bool is_k = !q_too || blockIdx.x >= BOUND_G;
+  const int blk = q_too && is_k ? blockIdx.x - BOUND_G : blockIdx.x;
   const uint16_t* base = (const uint16_t*)(is_k ? keys : p.q);  // keys: p.k, or one segment of the keys
   const int64_t sb = is_k ? p.ks_b : p.qs_b, sh = is_k ? p.ks_h : p.qs_h, ss = is_k ? p.ks_s : p.qs_s;
   const int S = is_k ? n_keys : p.Sq;
@@ -3380,7 +3382,7 @@ __global__ __launch_bounds__(256) void score_bound_partial_kernel(const AttnPara
     }
     __syncthreads();
   }
-  if (threadIdx.x == 0) part[blockIdx.x] = sm[0];
+  if (threadIdx.x == 0) part[is_k ? BOUND_G + blk : blk] = sm[0];
 }
 
 __global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part, int nparts, float scale_log2, float limit, int* flag) {
@@ -3388,7 +3390,7 @@ __global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part
   float mq = 0.f, mk = 0.f;
   for (int i = threadIdx.x; i < BOUND_G * nparts; i += 256) {  // nparts sets of (BOUND_G for Q, BOUND_G for a key segment)
     const int set = i / BOUND_G, e = i - set * BOUND_G;
-    mq = fmaxf(mq, part[2 * BOUND_G * set + e]);
+    if (set == 0) mq = fmaxf(mq, part[e]);  // the Q rows go with the first key segment only
     mk = fmaxf(mk, part[2 * BOUND_G * set + BOUND_G + e]);
   }
   sq[threadIdx.x] = mq;
@@ -3967,13 +3969,13 @@ static int launch_bound(const AttnParams& p, int dtype, int D, const KeySegs* se
     const int n_keys = segs ? segs->len : p.Skv;
     float* dst = part + (size_t)2 * BOUND_G * i;
     if (dtype == PA_DTYPE_BF16 && D == 128)
-      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 128>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 128>), dim3(i == 0 ? 2 * BOUND_G : BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys, i == 0 ? 1 : 0);
     else if (dtype == PA_DTYPE_BF16)
-      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 64>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+      hipLaunchKernelGGL((score_bound_partial_kernel<BF16, 64>), dim3(i == 0 ? 2 * BOUND_G : BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys, i == 0 ? 1 : 0);
     else if (D == 128)
-      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 128>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 128>), dim3(i == 0 ? 2 * BOUND_G : BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys, i == 0 ? 1 : 0);
     else
-      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 64>), dim3(2 * BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys);
+      hipLaunchKernelGGL((score_bound_partial_kernel<F16, 64>), dim3(i == 0 ? 2 * BOUND_G : BOUND_G), dim3(256), 0, st, p, dst, keys, n_keys, i == 0 ? 1 : 0);
     PA_CHECK_LAUNCH("score bound kernel");
   }
   hipLaunchKernelGGL(score_bound_flag_kernel, dim3(1), dim3(256), 0, st, (const float*)part, nseg, p.scale_log2, limit, flag);
