@@ -729,6 +729,33 @@ def test_random_configurations(cuda):
         _check(out, lse, ref_out, ref_lse, what)
 
 
+def test_short_key_kernel_random_configurations(cuda, tuning):
+    """Thirty seeded random draws for the kernel for short key sequences (forced on): batch, heads, query rows from a
+    handful to several query tiles per workgroup, 449..512 keys, dtype, scale, [B,H,S,D] or [B,S,H,D] memory for each
+    of q, k, v -- each against the fp64 oracle."""
+    tuning("short_keys", 1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rng = np.random.default_rng(77)
+    for case in range(30):
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 9))
+        big = rng.random() < 0.25  # now and then enough pieces for several per workgroup and runs that cross heads
+        Sq = int(rng.integers(256 * cus // (B * H), 3 * 256 * cus // (B * H))) if big else int(rng.integers(1, 1500))
+        Skv = int(rng.integers(449, 513))
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+        scale = None if rng.random() < 0.6 else float(rng.uniform(0.02, 0.3))
+        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=3000 + case, dtype=dtype)
+        heads = list(range(H)) if not big else sorted(set([0, H // 2, H - 1]))
+        rows = torch.arange(Sq) if not big else torch.cat([torch.arange(0, 300), torch.randint(0, Sq, (300,), generator=torch.Generator().manual_seed(case)), torch.arange(Sq - 300, Sq)])
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, heads][:, :, rows].float().numpy(), k[:, heads].float().numpy(), v[:, heads].float().numpy(), scale)
+        dev = [t.to(cuda) for t in (q, k, v)]
+        for i in range(3):
+            if rng.random() < 0.4:
+                dev[i] = dev[i].transpose(1, 2).contiguous().transpose(1, 2)
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(*dev, scale=scale)
+        _check(out[:, heads][:, :, rows.to(cuda)], lse[:, heads][:, :, rows.to(cuda)], ref_out, ref_lse,
+               f"case {case}: B{B} H{H} Sq{Sq} Skv{Skv} {dtype} scale={scale}")
+
+
 def test_key_rows_spread_over_4gib(cuda):
     """K and V whose rows lie 1 MiB apart span more than 4 GiB per head: beyond the 32-bit offsets of the
     pipelined kernel, so the launch must pick the kernel without that limit (a wrong pick reads zeros)."""
