@@ -59,6 +59,11 @@ PA_API const char* pa_last_error(void);
  *   "bound"        PARAATTN_BOUND=0|1       0 / 1: never / always compute the score bound, -1 = by size
  *   "stream"       PARAATTN_STREAM=0|1      0 / 1: never / wherever possible the kernel with resident workgroups, -1 = by shape
  *   "stream_even"  PARAATTN_STREAM_EVEN=0|1 that kernel's tail cut into shares that begin at the same keys / into equal ranges, -1 = by size
+ *   "stream_dyn"   PARAATTN_STREAM_DYN=0|2..6  that kernel's tail in equal ranges, one per workgroup / in that many rounds of ever
+ *                                           shorter ranges which the workgroups draw from a counter as they run out of work (so
+ *                                           that faster compute units take more), wherever two rounds fit; -1 = 4 rounds from 1024
+ *                                           key-tile steps per workgroup on.  Needs 4x the workspace of equal ranges; a call whose
+ *                                           workspace is smaller gets equal ranges.  Results do not depend on who drew what.
  *   "sparse_pair"  PARAATTN_SPARSE_PAIR=1   1: pa_attn_fwd_blocksparse with 128-row query blocks puts two adjacent blocks into one
  *                                           256-row workgroup that walks the union of their key ranges (head_dim 128)
  *   "wave_rows"    PARAATTN_WAVE_ROWS=64    64: the kernel with resident workgroups runs as 4 wavefronts of 64 query rows (one per SIMD,
@@ -168,9 +173,12 @@ PA_API size_t pa_attn_fwd_masked_workspace_bytes(int B, int H, int Sq, int Skv, 
  * PA_NOALLOC_SCRATCH_BYTES inside the library's device image, one copy per GPU,
  * held until the process ends; the call allocates and frees nothing.  Same
  * arguments, kernels and results as pa_attn_fwd_lse_ws with a workspace of
- * pa_attn_fwd_workspace_bytes() bytes.  A problem whose launch plan needs more
- * scratch than the buffer holds is refused with PA_ERR_WORKSPACE (it is not run
- * unsplit behind the caller's back).  Nothing in the buffer has to survive
+ * pa_attn_fwd_workspace_bytes() bytes, except that large problems (see the knob
+ * "stream_dyn") keep one tail range per workgroup, the plan pa_attn_fwd_lse_ws
+ * itself falls back to when its workspace is too small for drawn ranges; there
+ * the two entry points agree to rounding, not bit for bit.  A problem whose
+ * launch plan needs more scratch than the buffer holds even so is refused with
+ * PA_ERR_WORKSPACE (it is not run unsplit behind the caller's back).  Nothing in the buffer has to survive
  * between calls and nothing has to be cleared; but all calls on one GPU share
  * it, so calls that overlap on one GPU (two streams, two threads) race.
  */

@@ -59,10 +59,17 @@ constexpr float RESCALE_SLACK = 8.0f;
 // The keys of a piece may come in nseg segments of seg_len keys each (the blocks of a ring sweep), each with
 // its own base pointer and the strides of AttnParams.
 constexpr int MAX_KEY_SEGS = 16;
+constexpr int MAX_TAIL_ROUNDS = 6;
 struct StreamPlan {
   int G, R, Gt, L, n_pieces;
   int xcd_order;  // 1: workgroup numbers are dealt so that each of 8 XCDs holds a contiguous eighth of them
   int nseg, seg_len, tps;  // key segments, keys and key tiles per segment
+  // The tail's key-tile steps come in n_rounds rounds (steps round_at[r] .. round_at[r + 1] of the tail), each cut
+  // into Gt / n_rounds ranges of equal length.  next_range null: one round, range g belongs to workgroup g.
+  // Otherwise the ranges (rounds of G, ever shorter) are taken in turn from that counter, 0 before the launch.
+  int n_rounds;
+  int64_t round_at[MAX_TAIL_ROUNDS + 1];
+  int* next_range;
   const void* kseg[MAX_KEY_SEGS];
   const void* vseg[MAX_KEY_SEGS];
 };
@@ -1882,6 +1889,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   char* const sK = (char*)smem;                    // [2][64][256 B]
   char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
   char* const sStage = (char*)smem + 4 * TILE_BYTES;  // [NW wavefronts][WROWS rows][256 B]: finished outputs on their way out
+  int* const sTaken = (int*)((char*)smem + 4 * TILE_BYTES + 8 * 8192);  // the tail range that wavefront 0 drew for the workgroup
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1910,11 +1918,11 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   // R whole pieces, then one range of the tail's key-tile steps, which may run over several pieces.  The
   // generator walks items (piece, first tile, end tile) and inside an item the tiles, keeping (segment, tile
   // in segment).
-  int tail_left = 0;  // key tiles of this workgroup's tail range still to hand out
-  if (wg < sp.Gt) {
-    const int64_t Ttail = (int64_t)(sp.n_pieces - sp.R * sp.G) * sp.L;
-    tail_left = (int)((int64_t)(wg + 1) * Ttail / sp.Gt - (int64_t)wg * Ttail / sp.Gt);
-  }
+  // The tail's Gt ranges: without a counter, range wg belongs to this workgroup; with one, a workgroup that has run
+  // out of tiles draws the number of its next range from it, so the ranges go to whoever asks first (compute units
+  // do not all run at one speed: with equal shares the finish times of the workgroups were measured 7 % apart).
+  int tail_left = 0;  // key tiles of the current tail range still to hand out
+  int g_range = 0;    // the current range
   struct Desc {
     int piece;    // < 0: no such tile
     int flags;    // LAST: the item's last tile; FULL: the item is a whole piece; MID: the item begins inside a piece
@@ -1928,7 +1936,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
     g_piece = piece;
     g_j = j0;
     g_jend = jend;
-    g_kind = (j0 == 0 && jend == sp.L ? FULL : 0) | (j0 > 0 ? MID : 0);
+    g_kind = (j0 == 0 && jend == sp.L ? FULL : 0) | (j0 > 0 ? MID : 0) | (g_range << 3);
     g_seg = j0 / sp.tps;
     g_jj = j0 - g_seg * sp.tps;
   };
@@ -1946,12 +1954,36 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
       start_item(wg + g_round * G, 0, L);
       return true;
     }
-    if (tail_left <= 0) return false;
     int piece, j0;
-    if (!g_in_tail) {
+    if (tail_left <= 0) {  // the next range
+      const int Gt = kp->st.Gt;
+      int* const counter = kp->st.next_range;
+      int n;
+      if (counter != nullptr) {
+        // Every wavefront of the workgroup comes by here in the same iteration.  Wavefront 0 draws the number; the
+        // word it leaves in LDS is not written again before the next draw, at least 16 barriers later.
+        if (wave == 0) {
+          int v = 0;
+          if (lane == 0) v = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          *(volatile int*)sTaken = __builtin_amdgcn_readfirstlane(v);
+        }
+        __syncthreads();
+        n = __builtin_amdgcn_readfirstlane(*(volatile int*)sTaken);
+        if (n < 0) return false;
+      } else if (!g_in_tail) {
+        n = wg;
+      } else {
+        return false;
+      }
+      if (n >= Gt) return false;  // no range left
       g_in_tail = true;
-      const int64_t Ttail = (int64_t)(kp->st.n_pieces - R * G) * L;
-      const int64_t ta = (int64_t)wg * Ttail / kp->st.Gt;
+      g_range = n;
+      const int per_round = Gt / kp->st.n_rounds;
+      const int rd = n / per_round, i = n - rd * per_round;
+      const int64_t r0 = kp->st.round_at[rd], Tr = kp->st.round_at[rd + 1] - r0;
+      const int64_t ta = r0 + (int64_t)i * Tr / per_round;
+      tail_left = (int)(r0 + (int64_t)(i + 1) * Tr / per_round - ta);
+      if (tail_left <= 0) return false;
       piece = R * G + (int)(ta / L);
       j0 = (int)(ta % L);
     } else {
@@ -2168,7 +2200,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
           lse_out[((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row] = lse_nat;
       } else if (my_row < w.row_end) {
         if (!(d.flags & FULL)) {  // a share of a piece: normalised fp32 partial + LSE into the workspace
-          const int64_t wrow = (int64_t)(2 * wg + ((d.flags & MID) ? 0 : 1)) * 256 + (my_row - w.row_begin);
+          const int64_t wrow = (int64_t)(2 * (d.flags >> 3) + ((d.flags & MID) ? 0 : 1)) * 256 + (my_row - w.row_begin);
           float* wp = kp->ws_out + wrow * 128;
 #pragma unroll
           for (int db = 0; db < DB; ++db)
@@ -3054,9 +3086,14 @@ __global__ __launch_bounds__(256) void attn_stream_merge_kernel(const AttnParams
   const int local = ((blockIdx.x & 15) << 4) + (threadIdx.x >> 4);
   const int c8 = (threadIdx.x & 15) * 8;
   const int tail0 = sp.R * sp.G;
-  const int64_t Ttail = (int64_t)(sp.n_pieces - tail0) * sp.L;
-  // workgroup whose range holds tail step t: the largest g with g * Ttail / Gt <= t
-  auto slot = [&](int64_t t) { return (int)(((t + 1) * sp.Gt + Ttail - 1) / Ttail) - 1; };
+  // range that holds tail step t: in its round (of Tr steps from r0 on, cut into n ranges) the largest i with i * Tr / n <= t - r0
+  auto slot = [&](int64_t t) {
+    const int n = sp.Gt / sp.n_rounds;
+    int rd = 0;
+    while (rd + 1 < sp.n_rounds && t >= sp.round_at[rd + 1]) ++rd;
+    const int64_t r0 = sp.round_at[rd], Tr = sp.round_at[rd + 1] - r0;
+    return rd * n + (int)(((t - r0 + 1) * n + Tr - 1) / Tr) - 1;
+  };
   const int g_first = slot((int64_t)tp * sp.L), g_last = slot((int64_t)(tp + 1) * sp.L - 1);
   if (g_first == g_last) return;  // computed whole by one workgroup, which stored it itself
   const int piece = tail0 + tp;
@@ -3639,12 +3676,13 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
 //   PARAATTN_BOUND=0|1       "bound"         never / always compute the score bound (-1 = by size)
 //   PARAATTN_STREAM=0|1      "stream"        never / wherever possible the resident-workgroup kernel (-1 = by shape)
 //   PARAATTN_STREAM_EVEN=0|1 "stream_even"   its tail cut into shares that begin at the same keys / into equal ranges (-1 = by size)
+//   PARAATTN_STREAM_DYN=0|2..6 "stream_dyn"  its tail in equal ranges, one per workgroup / in that many rounds of ranges drawn by the workgroups, wherever two rounds fit (-1 = 4 rounds, by size)
 //   PARAATTN_SPARSE_PAIR=1   "sparse_pair"   block-sparse with 128-row query blocks: two adjacent blocks per 256-row workgroup
 //   PARAATTN_WAVE_ROWS=64    "wave_rows"     the resident-workgroup kernel as 4 wavefronts of 64 query rows instead of 8 of 32
 //   PARAATTN_SPARSE_ORDER=0  "sparse_order"  block-sparse: 0 = the query blocks of a head in their own order instead of longest list first
 //   PARAATTN_SHORT_KEYS=0|1  "short_keys"    never / wherever it applies the kernel for 449..512 keys (-1 = by the number of pieces)
 struct Tuning {
-  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, sparse_pair, wave_rows, short_keys, sparse_order;
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, stream_dyn, sparse_pair, wave_rows, short_keys, sparse_order;
 };
 static Tuning& tuning() {
   static Tuning t;
@@ -3663,6 +3701,8 @@ static Tuning& tuning() {
     t.stream = st == 0 || st == 1 ? st : -1;
     const int se = num("PARAATTN_STREAM_EVEN", -1);
     t.stream_even = se == 0 || se == 1 ? se : -1;
+    const int sd = num("PARAATTN_STREAM_DYN", -1);
+    t.stream_dyn = sd == 0 || (sd > 1 && sd <= MAX_TAIL_ROUNDS) ? sd : -1;
     t.sparse_pair = num("PARAATTN_SPARSE_PAIR", 0) == 1;
     t.wave_rows = num("PARAATTN_WAVE_ROWS", 0) == 64 ? 64 : 0;
     const int sk = num("PARAATTN_SHORT_KEYS", -1);
@@ -3686,6 +3726,7 @@ extern "C" int pa_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bound")) t.bound = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "stream")) t.stream = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "stream_even")) t.stream_even = value == 0 || value == 1 ? value : -1;
+  else if (!strcmp(name, "stream_dyn")) t.stream_dyn = value == 0 || (value > 1 && value <= MAX_TAIL_ROUNDS) ? value : -1;
   else if (!strcmp(name, "sparse_pair")) t.sparse_pair = value == 1;
   else if (!strcmp(name, "wave_rows")) t.wave_rows = value == 64 ? 64 : 0;
   else if (!strcmp(name, "short_keys")) t.short_keys = value == 0 || value == 1 ? value : -1;
@@ -3798,7 +3839,7 @@ struct KeySegs {
 // Plan for attn_fwd_d128_stream_kernel (see StreamPlan).  Returns false where that kernel does not apply or is
 // not expected to pay; otherwise fills p.st, p.bm, p.n_qtiles, and *ws_need with the bytes of workspace its
 // partial results take (0: no piece is cut).  `sizing`: report the plan that a sufficient workspace would get.
-static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_avail, bool sizing, size_t* ws_need) {
+static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_avail, bool sizing, size_t* ws_need, bool allow_drawn = true) {
   *ws_need = 0;
   const bool multi = segs != nullptr;
   const int want = tuning().stream;
@@ -3833,18 +3874,46 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   st.nseg = nseg;
   st.seg_len = seg_len;
   st.tps = tps;
+  st.next_range = nullptr;
+  st.n_rounds = 1;
+  st.round_at[0] = st.round_at[1] = 0;
   for (int i = 0; i < nseg; ++i) {
     st.kseg[i] = multi ? segs->k[i] : p.k;
     st.vseg[i] = multi ? segs->v[i] : p.v;
   }
-  const int p_tail = P - st.R * st.G;
+  // equal ranges by default: shares of whole pieces that begin at the same keys keep the tail's workgroups in step
+  // on the keys, but leave workgroups idle; measured slower or equal at every shape from 3000 to 119056 keys
+  const int ev = tuning().stream_even;
+  const bool even = ev != 0;
+  // Rounds of ever shorter ranges that go to whoever asks first (StreamPlan::next_range), from 1024 key-tile steps per
+  // workgroup on.  Workgroups given equal shares finish up to 7 % apart (some XCDs are slower than others, by box);
+  // drawn ranges bring that below 1 % and take 1.7 .. 2.9 % off the time of launches of 2.5 ms and more (119056 keys,
+  // Wan self-attention, a ring sweep, 16k tokens x 40 heads), but their 4 G partial results cost about 35 us to write
+  // and fold, which shorter launches do not earn back (measured +1 .. +8 % from 0.4 to 1.2 ms).
+  int dyn = 0;
+  if (allow_drawn && even && !tuning().no_split && (sizing || ws_avail > 0)) {
+    const int want_dyn = tuning().stream_dyn;
+    if (want_dyn > 1) dyn = want_dyn;
+    else if (want_dyn < 0 && (int64_t)P * L >= (int64_t)1024 * st.G) dyn = 4;
+  }
+  int p_tail = P - st.R * st.G;
+  if (dyn > 1) {
+    // they need a tail worth handing out, a twelfth of the work or more, and long enough for two rounds
+    int r = st.R, pt = p_tail;
+    while (r > 0 && (int64_t)pt * 12 < P) {
+      --r;
+      pt += st.G;
+    }
+    if ((int64_t)pt * L / 4 >= (int64_t)16 * st.G) {
+      st.R = r;
+      p_tail = pt;
+    } else {
+      dyn = 0;
+    }
+  }
   st.Gt = 0;
   if (p_tail > 0) {
     const int64_t t_tail = (int64_t)p_tail * L;
-    // equal ranges by default: shares of whole pieces that begin at the same keys keep the tail's workgroups in step
-    // on the keys, but leave workgroups idle; measured slower or equal at every shape from 3000 to 119056 keys
-    const int ev = tuning().stream_even;
-    const bool even = ev != 0;
     int gt;
     if (even) {
       const int64_t by_size = t_tail / 8;  // at least 8 key tiles per workgroup
@@ -3856,19 +3925,39 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
       if (sh < 1) sh = 1;
       gt = p_tail * sh;
     }
+    // rounds of G ranges, each round half of what is left (the last one all of it), none with ranges below 16 steps
+    int rounds = 1;
+    int64_t at[MAX_TAIL_ROUNDS + 1] = {0};
+    if (even && gt == st.G && dyn > 1) {
+      int64_t left = t_tail;
+      rounds = 0;
+      while (rounds + 1 < dyn && rounds + 1 < MAX_TAIL_ROUNDS && left / 4 >= (int64_t)16 * st.G) {
+        at[rounds + 1] = at[rounds] + left / 2;
+        left -= left / 2;
+        ++rounds;
+      }
+      ++rounds;  // the last round takes what is left
+      gt = rounds * st.G;
+    }
     if (tuning().no_split) gt = p_tail;
-    const size_t per_range = (size_t)2 * 256 * (128 + 1) * sizeof(float);  // two partial results per workgroup
-    size_t need = gt != p_tail ? gt * per_range : 0;
+    const size_t per_range = (size_t)2 * 256 * (128 + 1) * sizeof(float);  // two partial results per range
+    size_t need = gt != p_tail ? gt * per_range + (rounds > 1 ? 256 : 0) : 0;
+    if (need > ws_avail && !sizing && dyn > 1) return plan_stream(p, D, segs, ws_avail, sizing, ws_need, false);
     if (need > ws_avail && !sizing) {  // as many ranges as the workspace holds, if that still beats whole pieces
       const int64_t fit = (int64_t)(ws_avail / per_range);
       if (even && fit > p_tail) {
-        gt = (int)fit;
+        gt = (int)(fit < st.G ? fit : st.G);
         need = gt * per_range;
       } else {
         gt = p_tail;
         need = 0;
       }
     }
+    if (gt <= st.G) rounds = 1;
+    st.n_rounds = rounds;
+    for (int r = 1; r < rounds; ++r) st.round_at[r] = at[r];
+    st.round_at[0] = 0;
+    st.round_at[rounds] = t_tail;
     st.Gt = gt;
     *ws_need = need;
   }
@@ -3925,7 +4014,7 @@ static int launch_short(const AttnParams& p, hipStream_t stream) {
 
 template <typename T, int RB>
 static int launch_stream_rb(const AttnParams& p, hipStream_t stream) {
-  const size_t smem = 4 * TILE_BYTES + 8 * 8192;  // two K and two V tiles, and a staging area for outputs
+  const size_t smem = 4 * TILE_BYTES + 8 * 8192 + 16;  // two K and two V tiles, a staging area for outputs, two words
   static bool attr_done[PA_MAX_DEVICES][2] = {};  // benign race: the call is idempotent
   const int dev = current_device();
   for (int b = 0; b < 2; ++b) {
@@ -3945,9 +4034,18 @@ static int launch_stream_rb(const AttnParams& p, hipStream_t stream) {
   return PA_OK;
 }
 
+__global__ void clear_word_kernel(int* w, const int* gate, int gate_want) {
+  if (gate != nullptr && *gate != gate_want) return;
+  *w = 0;
+}
+
 template <typename T>
 static int launch_stream(const AttnParams& p, hipStream_t stream) {
   if (p.out == nullptr && p.acc_out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
+  if (p.st.next_range != nullptr) {  // a kernel, not a memset: the call may be under graph capture
+    hipLaunchKernelGGL(clear_word_kernel, dim3(1), dim3(1), 0, stream, p.st.next_range, p.gate, p.gate_want);
+    PA_CHECK_LAUNCH("range counter");
+  }
   const int rc = tuning().wave_rows == 64 ? launch_stream_rb<T, 2>(p, stream) : launch_stream_rb<T, 1>(p, stream);
   if (rc != PA_OK) return rc;
   const int p_tail = p.st.n_pieces - p.st.R * p.st.G;
@@ -4049,6 +4147,7 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
     if (stream_bytes > 0) {
       p.ws_out = (float*)ws_base;
       p.ws_lse = p.ws_out + (size_t)2 * p.st.Gt * 256 * 128;
+      if (p.st.n_rounds > 1) p.st.next_range = (int*)(ws_base + stream_bytes - 256);
     }
     if (B == 0 || H == 0 || Sq == 0) return PA_OK;
     return dtype == PA_DTYPE_BF16 ? launch_stream<BF16>(p, (hipStream_t)stream) : launch_stream<F16>(p, (hipStream_t)stream);
@@ -4134,7 +4233,8 @@ extern "C" size_t pa_attn_fwd_sweep_workspace_bytes(int B, int H, int Sq, int n_
 // with per-batch key counts (one workgroup per query tile, key-split tail); 2: the plan of an is_causal call
 // (never split: only the score bound's words); WS_ANY: the largest of them.
 constexpr int WS_ANY = 3;
-static size_t dense_ws_need(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3], const int64_t v_strides[3], int which) {
+static size_t dense_ws_need(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3], const int64_t v_strides[3], int which,
+                            bool allow_drawn = true) {
   const int64_t zero[3] = {0, 0, 0};
   size_t best = 0;
   for (int plan = 0; plan < 3; ++plan) {
@@ -4143,7 +4243,7 @@ static size_t dense_ws_need(int B, int H, int Sq, int Skv, int D, const int64_t 
     fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
     p.causal = plan == 2;
     size_t need = 0;
-    if (plan != 0 || !plan_stream(p, D, nullptr, 0, true, &need)) {
+    if (plan != 0 || !plan_stream(p, D, nullptr, 0, true, &need, allow_drawn)) {
       need = 0;
       choose_kernel(p, D, 256, true, 0, &need);
     }
@@ -4284,7 +4384,9 @@ extern "C" int pa_attn_fwd_lse_noalloc(const void* q, const void* k, const void*
                                        float scale, const int32_t* kv_len, int is_causal, void* stream) {
   // what the same problem would ask of a caller's workspace (0 for sizes that use none)
   const bool shaped = B > 0 && H > 0 && Sq > 0 && Skv > 0 && (D == 128 || D == 64) && k_strides && v_strides;
-  const size_t need = shaped ? dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, is_causal ? 2 : kv_len != nullptr ? 1 : 0) : 0;
+  // (the plan with one tail range per workgroup: the one a call falls back to when the workspace cannot hold the
+  // partial results of drawn ranges, which take four times as many)
+  const size_t need = shaped ? dense_ws_need(B, H, Sq, Skv, D, k_strides, v_strides, is_causal ? 2 : kv_len != nullptr ? 1 : 0, false) : 0;
   if (need > (size_t)PA_NOALLOC_SCRATCH_BYTES)
     PA_FAIL(PA_ERR_WORKSPACE, "this problem's launch plan needs %zu bytes of scratch, the static buffer holds %zu: "
             "call pa_attn_fwd_lse_ws with a workspace of your own", need, (size_t)PA_NOALLOC_SCRATCH_BYTES);

@@ -433,6 +433,81 @@ def test_resident_workgroup_kernel(cuda, even, bound, wave_rows, tuning):
     assert lib.pa_attn_fwd_workspace_bytes(1, 24, 4608, 4608, 128, _lib.strides3(qf), _lib.strides3(qf)) == 0
 
 
+@pytest.mark.parametrize("rounds", [2, 4, 6])
+@pytest.mark.parametrize("wave_rows", [32, 64])
+def test_resident_workgroups_draw_their_tail_ranges(cuda, rounds, wave_rows, tuning):
+    """The resident-workgroup kernel with its tail cut into rounds of ever shorter ranges that the workgroups draw
+    from a counter as they run out of work (by itself the planner does that from 1024 key-tile steps per workgroup
+    on; forced here at sizes the oracle can follow): fewer pieces than workgroups, a few pieces beyond a whole round,
+    and exactly two rounds of pieces (the plan then gives up a round of whole pieces to have a tail), ragged query
+    and key ends, both dtypes.  Sampled rows of three heads against the fp64 oracle; the whole output against the
+    plan with one range per workgroup; and bit for bit against a second call (which workgroup drew which range
+    differs from call to call and must not show)."""
+    import ctypes
+
+    from paraattention_amd import _lib
+
+    lib = _lib.load()
+    tuning("stream", 1)
+    tuning("wave_rows", wave_rows)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    op = torch.ops.para_attn.attention_forward_with_lse
+    shapes = [(1, 8, cus // 16 * 256 + 33, 64 * (260 if rounds > 2 else 130) + 7, torch.bfloat16),
+              (2, 5, (cus // 10 + 5) * 256 - 100, 64 * 400 + 1, torch.float16),
+              (1, 8, cus // 4 * 256, 64 * 70, torch.bfloat16)]
+    for B, H, Sq, Skv, dtype in shapes:
+        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=Sq + Skv, dtype=dtype)
+        qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+        tuning("stream_dyn", 0)
+        need0 = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, 128, _lib.strides3(kd), _lib.strides3(vd))
+        out0, lse0 = op(qd, kd, vd)
+        tuning("stream_dyn", rounds)
+        need = lib.pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, 128, _lib.strides3(kd), _lib.strides3(vd))
+        assert need >= 2 * cus * 2 * 256 * 129 * 4 > need0, "meant to take at least two rounds of ranges"
+        out, lse = op(qd, kd, vd)
+        heads = [0, H // 2, H - 1]
+        rows = torch.cat([torch.arange(0, 200), torch.randint(0, Sq, (200,), generator=torch.Generator().manual_seed(Sq)), torch.arange(Sq - 300, Sq)])
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, heads][:, :, rows].float().numpy(), k[:, heads].float().numpy(), v[:, heads].float().numpy())
+        _check(out[:, heads][:, :, rows.to(cuda)], lse[:, heads][:, :, rows.to(cuda)], ref_out, ref_lse, f"drawn ranges {(B, H, Sq, Skv, dtype)} rounds={rounds}")
+        assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
+        for _ in range(2):
+            out2, lse2 = op(qd, kd, vd)
+            assert torch.equal(out2, out) and torch.equal(lse2, lse)
+        # a workspace that holds the equal ranges but not the drawn ones: the call falls back to the former
+        ws = torch.empty(need0, dtype=torch.uint8, device=cuda)
+        out3, lse3 = torch.empty_like(qd), torch.empty_like(lse)
+        vp = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+        rc = lib.pa_attn_fwd_lse_ws(vp(qd), vp(kd), vp(vd), vp(out3), vp(lse3), 0 if dtype == torch.bfloat16 else 1, B, H, Sq, Skv, 128,
+                                    _lib.strides3(qd), _lib.strides3(kd), _lib.strides3(vd), _lib.strides3(out3), 1.0 / math.sqrt(128), None, 0,
+                                    vp(ws), need0, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.pa_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(out3, out0) and torch.equal(lse3, lse0)
+
+
+def test_planner_draws_ranges_for_long_launches_only(cuda, tuning):
+    """What the planner asks of the workspace says which plan it took: four rounds of ranges (4 x compute units x two
+    partial results, and the counter's 256 bytes) from 1024 key-tile steps per workgroup on, at most one range per
+    workgroup below."""
+    import ctypes
+
+    from paraattention_amd import _lib
+
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    tuning("bound", 0)
+    per_range = 2 * 256 * 129 * 4
+
+    def need(H, S):
+        st = (ctypes.c_int64 * 3)(H * S * 128, S * 128, 128)
+        return lib.pa_attn_fwd_workspace_bytes(1, H, S, S, 128, st, st)
+
+    assert need(3, 119056) == 4 * cus * per_range + 256
+    assert need(40, 32760) == 4 * cus * per_range + 256
+    assert need(24, 4608) <= cus * per_range
+    assert need(24, 8192) <= cus * per_range
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_short_key_kernel(cuda, dtype, tuning):
     """The kernel for 449..512 keys per head (cross-attention to a text prompt), forced on for every shape here:
