@@ -38,9 +38,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Traffic at the L2's memory side per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two
 # rocprofv3 --pmc runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy).  These counters cannot be
 # read from inside this process; the figures are those of the summary named in TRAFFIC_SOURCE, not of this run.
-TRAFFIC = {"attn": 9.750e9, "merge": 4.773e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 9.193e9,
-           "flux": 3.012e8, "ring_sweep": 1.224e10, "ring_sweep_per_block": 1.509e10, "wan_self": 3.360e9, "wan_cross": 7.012e8,
-           "causal": 5.161e9, "head_dim_64": 2.438e9}
+TRAFFIC = {"attn": 1.006e10, "merge": 4.771e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 9.250e9,
+           "flux": 3.017e8, "ring_sweep": 1.234e10, "ring_sweep_per_block": 1.436e10, "wan_self": 3.745e9, "wan_cross": 7.018e8,
+           "causal": 5.160e9, "head_dim_64": 2.438e9}
 TRAFFIC_SOURCE = "profiles/kernels_bench_workloads.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the same command)"
 
 
