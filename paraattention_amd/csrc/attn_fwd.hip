@@ -50,12 +50,13 @@ constexpr float RESCALE_SLACK = 8.0f;
 // Work plan of attn_fwd_d128_stream_kernel.  The launch has G workgroups of 256 query rows that stay resident.
 // A piece is one query tile of one (batch, head) with its L key tiles.  Workgroup g first computes the R whole
 // pieces g, g + G, ..., all workgroups sweeping the keys in step (so a K/V tile is fetched once per L2 and
-// round); what is left, fewer than G pieces, is a list of (n_pieces - R G) L key-tile steps cut into Gt equal
-// ranges, one for each of the first Gt workgroups.  A range that does not cover a whole piece leaves a
-// normalised fp32 partial result and its LSE in the workspace (at most two per workgroup: row 2g for a share
-// that begins inside a piece, 2g + 1 for one that begins a piece but does not finish it), which
-// attn_stream_merge_kernel folds.  Gt = G cuts the tail evenly; Gt = (pieces left) x s cuts every piece
-// left into s shares that begin at the same keys.
+// round); what is left (fewer than G pieces, or more where the plan keeps rounds of pieces back for it) is a list
+// of (n_pieces - R G) L key-tile steps cut into Gt ranges: one for each of the first Gt workgroups, or, for long
+// launches, rounds of ever shorter ranges that the workgroups draw from a counter as they run out of work.  A
+// range that does not cover a whole piece leaves a normalised fp32 partial result and its LSE in the workspace
+// (at most two per range: row 2n for a share that begins inside a piece, 2n + 1 for one that begins a piece but
+// does not finish it), which attn_stream_merge_kernel folds.  Gt = G cuts the tail evenly; Gt = (pieces left) x s
+// cuts every piece left into s shares that begin at the same keys.
 // The keys of a piece may come in nseg segments of seg_len keys each (the blocks of a ring sweep), each with
 // its own base pointer and the strides of AttnParams.
 constexpr int MAX_KEY_SEGS = 16;
