@@ -64,6 +64,8 @@ PA_API const char* pa_last_error(void);
  *                                           that faster compute units take more), wherever two rounds fit; -1 = 4 rounds from 1024
  *                                           key-tile steps per workgroup on.  Needs 4x the workspace of equal ranges; a call whose
  *                                           workspace is smaller gets equal ranges.  Results do not depend on who drew what.
+ *   "stream_solo"  PARAATTN_STREAM_SOLO=1   test aid: a launch all of whose pieces are cut into drawn ranges (fewer pieces than
+ *                                           compute units) is computed by one workgroup, which draws every range in turn
  *   "sparse_pair"  PARAATTN_SPARSE_PAIR=1   1: pa_attn_fwd_blocksparse with 128-row query blocks puts two adjacent blocks into one
  *                                           256-row workgroup that walks the union of their key ranges (head_dim 128)
  *   "wave_rows"    PARAATTN_WAVE_ROWS=64    64: the kernel with resident workgroups runs as 4 wavefronts of 64 query rows (one per SIMD,

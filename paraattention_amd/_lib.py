@@ -147,7 +147,7 @@ def check(rc, what):
 
 def set_tuning(name, value):
     """Set one tuning / test knob of the attention launches (pa_set_tuning in the header): "no_pipe", "bm",
-    "no_split", "no_xcd_order", "bound", "stream", "stream_even", "stream_dyn", "sparse_pair", "wave_rows", "short_keys", "sparse_order".  The PARAATTN_* environment variables only give the initial values."""
+    "no_split", "no_xcd_order", "bound", "stream", "stream_even", "stream_dyn", "stream_solo", "sparse_pair", "wave_rows", "short_keys", "sparse_order".  The PARAATTN_* environment variables only give the initial values."""
     check(load().pa_set_tuning(name.encode(), int(value)), "pa_set_tuning")
 
 

@@ -71,6 +71,7 @@ struct StreamPlan {
   int n_rounds;
   int64_t round_at[MAX_TAIL_ROUNDS + 1];
   int* next_range;
+  int solo;  // test aid, with next_range and R = 0 only: workgroup 0 draws and computes every range, the others leave
   const void* kseg[MAX_KEY_SEGS];
   const void* vseg[MAX_KEY_SEGS];
 };
@@ -1902,6 +1903,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   // workgroup numbers, so the pieces its 32 workgroups sweep at one time are neighbours (one or two heads, whose
   // K/V tiles then meet in that XCD's L2), and so are its ranges of the tail.
   const int wg = sp.xcd_order ? (int)(blockIdx.x & 7) * (sp.G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  if (sp.solo && wg != 0) return;
   constexpr uint32_t OOB = PIPE_OOB;
   // What happens once per piece (a new Q, a new K/V descriptor, a finished piece's output) needs many of the
   // kernel's arguments and little else.  Read through `p` the compiler would load them all once, ahead of the
@@ -2617,6 +2619,8 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   // the first key only).
   auto inside_run = [&]() __attribute__((always_inline)) {
     if (nx2.piece < 0 || cur.piece != nx2.piece || cur.seg != nx2.seg || g_jj == 0) return 0;
+    // (two items in a row can belong to one piece: a workgroup that draws the range after its own)
+    if ((cur.flags | nxt.flags) & LAST) return 0;
     const int a = g_jend - 1 - g_j, b = sp.tps - 1 - g_jj;
     const int n = a < b ? a : b;
     return n > 0 ? n : 0;
@@ -3678,12 +3682,13 @@ static SplitPlan plan_split(int64_t n_tiles, int slots, int kv_tiles, int bm, bo
 //   PARAATTN_STREAM=0|1      "stream"        never / wherever possible the resident-workgroup kernel (-1 = by shape)
 //   PARAATTN_STREAM_EVEN=0|1 "stream_even"   its tail cut into shares that begin at the same keys / into equal ranges (-1 = by size)
 //   PARAATTN_STREAM_DYN=0|2..6 "stream_dyn"  its tail in equal ranges, one per workgroup / in that many rounds of ranges drawn by the workgroups, wherever two rounds fit (-1 = 4 rounds, by size)
+//   PARAATTN_STREAM_SOLO=1   "stream_solo"   test aid: where every piece is cut into drawn ranges, one workgroup draws and computes them all, one after the other
 //   PARAATTN_SPARSE_PAIR=1   "sparse_pair"   block-sparse with 128-row query blocks: two adjacent blocks per 256-row workgroup
 //   PARAATTN_WAVE_ROWS=64    "wave_rows"     the resident-workgroup kernel as 4 wavefronts of 64 query rows instead of 8 of 32
 //   PARAATTN_SPARSE_ORDER=0  "sparse_order"  block-sparse: 0 = the query blocks of a head in their own order instead of longest list first
 //   PARAATTN_SHORT_KEYS=0|1  "short_keys"    never / wherever it applies the kernel for 449..512 keys (-1 = by the number of pieces)
 struct Tuning {
-  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, stream_dyn, sparse_pair, wave_rows, short_keys, sparse_order;
+  std::atomic<int> no_pipe, no_split, no_xcd_order, forced_bm, bound, stream, stream_even, stream_dyn, stream_solo, sparse_pair, wave_rows, short_keys, sparse_order;
 };
 static Tuning& tuning() {
   static Tuning t;
@@ -3704,6 +3709,7 @@ static Tuning& tuning() {
     t.stream_even = se == 0 || se == 1 ? se : -1;
     const int sd = num("PARAATTN_STREAM_DYN", -1);
     t.stream_dyn = sd == 0 || (sd > 1 && sd <= MAX_TAIL_ROUNDS) ? sd : -1;
+    t.stream_solo = num("PARAATTN_STREAM_SOLO", 0) == 1;
     t.sparse_pair = num("PARAATTN_SPARSE_PAIR", 0) == 1;
     t.wave_rows = num("PARAATTN_WAVE_ROWS", 0) == 64 ? 64 : 0;
     const int sk = num("PARAATTN_SHORT_KEYS", -1);
@@ -3728,6 +3734,7 @@ extern "C" int pa_set_tuning(const char* name, int value) {
   else if (!strcmp(name, "stream")) t.stream = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "stream_even")) t.stream_even = value == 0 || value == 1 ? value : -1;
   else if (!strcmp(name, "stream_dyn")) t.stream_dyn = value == 0 || (value > 1 && value <= MAX_TAIL_ROUNDS) ? value : -1;
+  else if (!strcmp(name, "stream_solo")) t.stream_solo = value == 1;
   else if (!strcmp(name, "sparse_pair")) t.sparse_pair = value == 1;
   else if (!strcmp(name, "wave_rows")) t.wave_rows = value == 64 ? 64 : 0;
   else if (!strcmp(name, "short_keys")) t.short_keys = value == 0 || value == 1 ? value : -1;
@@ -3876,6 +3883,7 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   st.seg_len = seg_len;
   st.tps = tps;
   st.next_range = nullptr;
+  st.solo = 0;
   st.n_rounds = 1;
   st.round_at[0] = st.round_at[1] = 0;
   for (int i = 0; i < nseg; ++i) {
@@ -4148,7 +4156,10 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
     if (stream_bytes > 0) {
       p.ws_out = (float*)ws_base;
       p.ws_lse = p.ws_out + (size_t)2 * p.st.Gt * 256 * 128;
-      if (p.st.n_rounds > 1) p.st.next_range = (int*)(ws_base + stream_bytes - 256);
+      if (p.st.n_rounds > 1) {
+        p.st.next_range = (int*)(ws_base + stream_bytes - 256);
+        p.st.solo = tuning().stream_solo && p.st.R == 0;
+      }
     }
     if (B == 0 || H == 0 || Sq == 0) return PA_OK;
     return dtype == PA_DTYPE_BF16 ? launch_stream<BF16>(p, (hipStream_t)stream) : launch_stream<F16>(p, (hipStream_t)stream);

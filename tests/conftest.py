@@ -21,7 +21,7 @@ def cuda():
     return torch.device("cuda:0")
 
 
-_KNOB_DEFAULTS = {"no_pipe": 0, "bm": 0, "no_split": 0, "no_xcd_order": 0, "bound": -1, "stream": -1, "stream_even": -1, "stream_dyn": -1, "sparse_pair": 0, "wave_rows": 0, "short_keys": -1, "sparse_order": 1}
+_KNOB_DEFAULTS = {"no_pipe": 0, "bm": 0, "no_split": 0, "no_xcd_order": 0, "bound": -1, "stream": -1, "stream_even": -1, "stream_dyn": -1, "stream_solo": 0, "sparse_pair": 0, "wave_rows": 0, "short_keys": -1, "sparse_order": 1}
 
 
 @pytest.fixture

@@ -101,12 +101,12 @@ def test_tuning_knobs_are_validated():
         assert lib.pa_set_tuning(b"bm", 100) == _lib.PA_ERR_INVALID and b"bm" in lib.pa_last_error()
         assert lib.pa_set_tuning(b"no_such_knob", 1) == _lib.PA_ERR_INVALID
         assert lib.pa_set_tuning(None, 1) == _lib.PA_ERR_INVALID
-        for name in (b"no_pipe", b"no_split", b"no_xcd_order", b"bound", b"stream", b"stream_even", b"stream_dyn", b"sparse_pair", b"wave_rows", b"short_keys", b"sparse_order"):
+        for name in (b"no_pipe", b"no_split", b"no_xcd_order", b"bound", b"stream", b"stream_even", b"stream_dyn", b"stream_solo", b"sparse_pair", b"wave_rows", b"short_keys", b"sparse_order"):
             assert lib.pa_set_tuning(name, 1) == _lib.PA_OK
         with pytest.raises(ValueError):
             _lib.set_tuning("bm", 64)
     finally:
-        for name, val in (("no_pipe", 0), ("bm", 0), ("no_split", 0), ("no_xcd_order", 0), ("bound", -1), ("stream", -1), ("stream_even", -1), ("stream_dyn", -1), ("sparse_pair", 0), ("wave_rows", 0), ("short_keys", -1), ("sparse_order", 1)):
+        for name, val in (("no_pipe", 0), ("bm", 0), ("no_split", 0), ("no_xcd_order", 0), ("bound", -1), ("stream", -1), ("stream_even", -1), ("stream_dyn", -1), ("stream_solo", 0), ("sparse_pair", 0), ("wave_rows", 0), ("short_keys", -1), ("sparse_order", 1)):
             _lib.set_tuning(name, val)
 
 

@@ -485,6 +485,35 @@ def test_resident_workgroups_draw_their_tail_ranges(cuda, rounds, wave_rows, tun
         assert torch.equal(out3, out0) and torch.equal(lse3, lse0)
 
 
+@pytest.mark.parametrize("rounds", [2, 5])
+@pytest.mark.parametrize("wave_rows", [32, 64])
+def test_one_workgroup_draws_every_range(cuda, rounds, wave_rows, tuning):
+    """A workgroup may draw the range that follows its own: two items in a row then belong to one piece (no new Q, no
+    new K/V descriptor), and the first one's partial result must still be written and the accumulators cleared before
+    the second begins.  With 256 workgroups drawing at once that is rare; the test aid `stream_solo` has workgroup 0
+    draw and compute every range in turn, so every boundary between ranges is of that kind.  Fewer pieces than
+    compute units (all work is in the tail); against the fp64 oracle and the plan with one range per workgroup."""
+    tuning("stream", 1)
+    tuning("wave_rows", wave_rows)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    op = torch.ops.para_attn.attention_forward_with_lse
+    B, H, Sq, Skv = 1, 4, cus // 16 * 256 + 33, 64 * 520 + 7
+    q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=5)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    tuning("stream_dyn", 0)
+    out0, lse0 = op(qd, kd, vd)
+    tuning("stream_dyn", rounds)
+    tuning("stream_solo", 1)
+    out, lse = op(qd, kd, vd)
+    rows = torch.cat([torch.arange(0, 300), torch.arange(Sq - 300, Sq)])
+    ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), k.float().numpy(), v.float().numpy())
+    _check(out[:, :, rows.to(cuda)], lse[:, :, rows.to(cuda)], ref_out, ref_lse, f"one workgroup, {rounds} rounds")
+    assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
+    tuning("stream_solo", 0)
+    out2, lse2 = op(qd, kd, vd)  # the same ranges drawn by all workgroups: the same bits
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+
+
 def test_planner_draws_ranges_for_long_launches_only(cuda, tuning):
     """What the planner asks of the workspace says which plan it took: four rounds of ranges (4 x compute units x two
     partial results, and the counter's 256 bytes) from 1024 key-tile steps per workgroup on, at most one range per
