@@ -72,6 +72,7 @@ struct StreamPlan {
   int64_t round_at[MAX_TAIL_ROUNDS + 1];
   int* next_range;
   int solo;  // test aid, with next_range and R = 0 only: workgroup 0 draws and computes every range, the others leave
+  int has_kvlen;  // AttnParams.kv_len is set: a piece ends at its batch element's key count (one key segment only)
   const void* kseg[MAX_KEY_SEGS];
   const void* vseg[MAX_KEY_SEGS];
 };
@@ -1877,7 +1878,7 @@ static_assert(rb2_steps_meet_deadlines(), "softmax steps are dealt too late for 
 // the long shapes (the kernel sits at the chip's power limit either way: 68 % MFMA occupancy at 1.72 GHz
 // against 74 % at 1.60 GHz) and slower on short pieces, so it stays behind the "wave_rows" knob.
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool BOUNDED, int RB = 1>
+template <typename T, bool BOUNDED, int RB = 1, bool KVLEN = false>
 __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
   static_assert(RB == 1 || RB == 2, "a wavefront owns 32 or 64 query rows");
@@ -1917,6 +1918,21 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
     return kp;
   };
 
+  // ---- per-piece facts ---------------------------------------------------------------------------
+  struct Where {
+    int batch, head, row_begin, row_end;
+  };
+  auto where = [&](KArgs kp, int piece) __attribute__((always_inline)) {
+    Where w;
+    const int nqt = kp->n_qtiles, H = kp->H, Sq = kp->Sq;
+    const int bh = piece / nqt;
+    const int qt = piece - bh * nqt;
+    w.head = bh % H;
+    w.batch = bh / H;
+    w.row_begin = qt * 256;
+    w.row_end = w.row_begin + 256 < Sq ? w.row_begin + 256 : Sq;
+    return w;
+  };
   // ---- this workgroup's list of key tiles ------------------------------------------------------
   // R whole pieces, then one range of the tail's key-tile steps, which may run over several pieces.  The
   // generator walks items (piece, first tile, end tile) and inside an item the tiles, keeping (segment, tile
@@ -1935,19 +1951,64 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   constexpr int LAST = 1, FULL = 2, MID = 4;
   int g_round = -1, g_piece = 0, g_j = 0, g_kind = 0, g_jend = 0, g_seg = 0, g_jj = 0;
   bool g_in_tail = false, g_done = false;
+  // A variant of its own: in one kernel the paths it adds cost the plain calls 0.3 %.  Inside the variant the test
+  // stays a run-time one on purpose: as a compile-time constant the same code came out with spills in the hot loop
+  // (17.3 ms against 16.6 ms for the 119k-token call with a text-padding mask).
+  const bool has_kvlen = KVLEN && sp.has_kvlen != 0;
+  // keys of a piece: its batch element's count where the call gives per-batch key counts, else all of the segment's
+  auto key_limit = [&](int piece) __attribute__((always_inline)) {
+    const KArgs kp = kargs();
+    const int n = kp->kv_len[where(kp, piece).batch], all = kp->st.seg_len;
+    return n < 0 ? 0 : n < all ? n : all;
+  };
+  // An item is a run of key tiles of one piece.  With per-batch key counts it ends where the piece's keys end and
+  // may come out empty (g_j >= g_jend): see write_empty.
   auto start_item = [&](int piece, int j0, int jend) __attribute__((always_inline)) {
     g_piece = piece;
+    g_kind = (j0 == 0 && jend == sp.L ? FULL : 0) | (j0 > 0 ? MID : 0) | (g_range << 3);
+    if (has_kvlen) {
+      const int tiles = (key_limit(piece) + BN - 1) / BN;
+      jend = jend < tiles ? jend : tiles;
+    }
     g_j = j0;
     g_jend = jend;
-    g_kind = (j0 == 0 && jend == sp.L ? FULL : 0) | (j0 > 0 ? MID : 0) | (g_range << 3);
     g_seg = j0 / sp.tps;
     g_jj = j0 - g_seg * sp.tps;
   };
-  // valid keys of the tile that begins at key n0 of its segment (0 for a tile that does not exist)
-  auto valid_keys = [&](uint32_t n0) __attribute__((always_inline)) {
-    if (n0 == OOB) return 0;
-    const int left = sp.seg_len - (int)n0;
+  // valid keys of a tile (0 for a tile that does not exist)
+  auto valid_keys = [&](const Desc& d) __attribute__((always_inline)) {
+    if (d.n0 == OOB) return 0;
+    const int left = (has_kvlen ? key_limit(d.piece) : sp.seg_len) - (int)d.n0;
     return left < BN ? left : BN;
+  };
+  // The result of an item without keys, written where finish_item would write it: zeros and an LSE of -inf, as the
+  // output of a whole piece or as a partial result (whose row the fold kernel reads whatever it holds).
+  auto write_empty = [&]() __attribute__((always_inline)) {
+    const KArgs kp = kargs();
+    const Where w = where(kp, g_piece);
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int l32 = ln & 31, hh = ln >> 5;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int my_row = w.row_begin + wave * WROWS + 32 * rb + l32;
+      if (my_row >= w.row_end) continue;
+      if (g_kind & FULL) {
+        uint16_t* op = (uint16_t*)kp->out + w.batch * kp->os_b + w.head * kp->os_h + (int64_t)my_row * kp->os_s + 64 * hh;
+        const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) *(u32x4*)(op + 8 * i) = z;
+        float* const lse_out = kp->lse;
+        if (lse_out != nullptr && hh == 0) lse_out[((int64_t)w.batch * kp->H + w.head) * kp->Sq + my_row] = -INFINITY;
+      } else {
+        const int64_t wrow = (int64_t)(2 * (g_kind >> 3) + ((g_kind & MID) ? 0 : 1)) * 256 + (my_row - w.row_begin);
+        float* wp = kp->ws_out + wrow * 128 + 64 * hh;
+        const float4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 16; ++i) *(float4*)(wp + 4 * i) = z;
+        if (hh == 0) kp->ws_lse[wrow] = -INFINITY;
+      }
+    }
   };
   auto advance_item = [&]() __attribute__((always_inline)) -> bool {
     const KArgs kp = kargs();
@@ -1999,7 +2060,14 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
     return true;
   };
   auto pull = [&](Desc& d) __attribute__((always_inline)) {
-    if (!g_done && g_j >= g_jend) g_done = !advance_item();
+    if (!g_done && g_j >= g_jend) {
+      g_done = !advance_item();
+      if (has_kvlen)
+        while (!g_done && g_j >= g_jend) {  // an item beyond its piece's keys
+          write_empty();
+          g_done = !advance_item();
+        }
+    }
     if (g_done) {
       d.piece = -1; d.flags = 0; d.seg = 0; d.n0 = OOB;
       return;
@@ -2020,21 +2088,6 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   pull(nx2);
   if (cur.piece < 0) return;  // nothing for this workgroup (before any barrier: the whole workgroup leaves)
 
-  // ---- per-piece facts ---------------------------------------------------------------------------
-  struct Where {
-    int batch, head, row_begin, row_end;
-  };
-  auto where = [&](KArgs kp, int piece) __attribute__((always_inline)) {
-    Where w;
-    const int nqt = kp->n_qtiles, H = kp->H, Sq = kp->Sq;
-    const int bh = piece / nqt;
-    const int qt = piece - bh * nqt;
-    w.head = bh % H;
-    w.batch = bh / H;
-    w.row_begin = qt * 256;
-    w.row_end = w.row_begin + 256 < Sq ? w.row_begin + 256 : Sq;
-    return w;
-  };
   vec8 qf[RB][DC];  // B operand of the first GEMM: the Q rows of the piece whose scores are computed next
   auto load_q = [&](int piece) __attribute__((always_inline)) {
     const KArgs kp = kargs();
@@ -2304,7 +2357,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
     for (int rb = 0; rb < RB; ++rb) sn[rb][1] = T::mfma32(f[dc], qf[rb][dc], sn[rb][1]);
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const int nv0 = valid_keys(cur.n0);
+    const int nv0 = valid_keys(cur);
     if (nv0 < BN) mask_tail(sn[rb][0], sn[rb][1], nv0);
     if constexpr (!BOUNDED) {
       float m2 = fmaxf(sn[rb][0][0], sn[rb][1][0]);
@@ -2391,7 +2444,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (!inside) {
-        const int nv1 = valid_keys(nxt.n0);
+        const int nv1 = valid_keys(nxt);
         if (nv1 < BN) mask_tail(sn[0][0], sn[0][1], nv1);  // ragged or absent tile j+1
         // Q of the piece after next takes over the registers, if tile j+2 opens another piece than tile j+1
         if (nx2.piece >= 0 && nx2.piece != nxt.piece) load_q(nx2.piece);
@@ -2549,7 +2602,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
         }
       }
       if constexpr (!inside) {
-        const int nv1 = valid_keys(nxt.n0);
+        const int nv1 = valid_keys(nxt);
         if (nv1 < BN) {  // ragged or absent tile j+1
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) mask_tail(sn[rb][0], sn[rb][1], nv1);
@@ -3456,10 +3509,10 @@ __global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part
 // counts as kv_len and the mask need not be looked at again).  One workgroup; out[0..B) = counts,
 // out[B] = 1 if all are prefixes else 0.
 __global__ __launch_bounds__(1024) void key_mask_scan_kernel(const uint8_t* mask, int64_t mb, int64_t mk, int B,
-                                                             int Skv, int32_t* out) {
+                                                             int Skv, int32_t* out, int tell_nearly_all) {
   __shared__ int s_cnt[1024];
   __shared__ int s_last[1024];
-  int all_prefix = 1;
+  int all_prefix = 1, fewest = Skv;
   for (int b = 0; b < B; ++b) {
     int cnt = 0, last = -1;
     for (int j = threadIdx.x; j < Skv; j += 1024) {
@@ -3480,9 +3533,11 @@ __global__ __launch_bounds__(1024) void key_mask_scan_kernel(const uint8_t* mask
     }
     if (threadIdx.x == 0) out[b] = s_cnt[0];
     if (s_cnt[0] != s_last[0] + 1) all_prefix = 0;
+    fewest = min(fewest, s_cnt[0]);
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[B] = all_prefix;
+  // 0: not prefixes; 1: prefixes; 2 (where asked for): prefixes that keep at least 7/8 of the keys in every batch element
+  if (threadIdx.x == 0) out[B] = !all_prefix ? 0 : tell_nearly_all && (int64_t)fewest * 8 >= (int64_t)Skv * 7 ? 2 : 1;
 }
 
 }  // namespace pa
@@ -3847,12 +3902,16 @@ struct KeySegs {
 // Plan for attn_fwd_d128_stream_kernel (see StreamPlan).  Returns false where that kernel does not apply or is
 // not expected to pay; otherwise fills p.st, p.bm, p.n_qtiles, and *ws_need with the bytes of workspace its
 // partial results take (0: no piece is cut).  `sizing`: report the plan that a sufficient workspace would get.
-static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_avail, bool sizing, size_t* ws_need, bool allow_drawn = true) {
+static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_avail, bool sizing, size_t* ws_need, bool allow_drawn = true,
+                        bool allow_kvlen = false) {
   *ws_need = 0;
   const bool multi = segs != nullptr;
   const int want = tuning().stream;
   if (want == 0 || (want < 0 && tuning().forced_bm != 0)) return false;  // switched off, or a workgroup size of the other kernels asked for
-  if (D != 128 || p.causal || p.kv_len != nullptr || tuning().no_pipe) return false;
+  // per-batch key counts: only for a caller who knows that they leave nearly all keys (the plan is made for all of
+  // them, and pieces that end early leave their workgroups idle), one key segment
+  if (p.kv_len != nullptr && (!allow_kvlen || multi)) return false;
+  if (D != 128 || p.causal || tuning().no_pipe) return false;
   const int cus = device_cus();
   if (cus <= 0) return false;
   const int seg_len = multi ? segs->len : p.Skv, nseg = multi ? segs->n : 1;
@@ -3884,6 +3943,7 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   st.tps = tps;
   st.next_range = nullptr;
   st.solo = 0;
+  st.has_kvlen = p.kv_len != nullptr;
   st.n_rounds = 1;
   st.round_at[0] = st.round_at[1] = 0;
   for (int i = 0; i < nseg; ++i) {
@@ -3951,7 +4011,7 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
     if (tuning().no_split) gt = p_tail;
     const size_t per_range = (size_t)2 * 256 * (128 + 1) * sizeof(float);  // two partial results per range
     size_t need = gt != p_tail ? gt * per_range + (rounds > 1 ? 256 : 0) : 0;
-    if (need > ws_avail && !sizing && dyn > 1) return plan_stream(p, D, segs, ws_avail, sizing, ws_need, false);
+    if (need > ws_avail && !sizing && dyn > 1) return plan_stream(p, D, segs, ws_avail, sizing, ws_need, false, allow_kvlen);
     if (need > ws_avail && !sizing) {  // as many ranges as the workspace holds, if that still beats whole pieces
       const int64_t fit = (int64_t)(ws_avail / per_range);
       if (even && fit > p_tail) {
@@ -4021,7 +4081,7 @@ static int launch_short(const AttnParams& p, hipStream_t stream) {
   return PA_OK;
 }
 
-template <typename T, int RB>
+template <typename T, int RB, bool KVLEN>
 static int launch_stream_rb(const AttnParams& p, hipStream_t stream) {
   const size_t smem = 4 * TILE_BYTES + 8 * 8192 + 16;  // two K and two V tiles, a staging area for outputs, two words
   static bool attr_done[PA_MAX_DEVICES][2] = {};  // benign race: the call is idempotent
@@ -4029,16 +4089,16 @@ static int launch_stream_rb(const AttnParams& p, hipStream_t stream) {
   for (int b = 0; b < 2; ++b) {
     if (b == 1 && p.bound_flag == nullptr) break;
     if (dev >= 0 && attr_done[dev][b]) continue;
-    const void* fn = b ? (const void*)attn_fwd_d128_stream_kernel<T, true, RB> : (const void*)attn_fwd_d128_stream_kernel<T, false, RB>;
+    const void* fn = b ? (const void*)attn_fwd_d128_stream_kernel<T, true, RB, KVLEN> : (const void*)attn_fwd_d128_stream_kernel<T, false, RB, KVLEN>;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) PA_FAIL(PA_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     if (dev >= 0) attr_done[dev][b] = true;
   }
   if (p.bound_flag != nullptr) {  // one of the two variants leaves at once
-    hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, true, RB>), dim3((unsigned)p.st.G), dim3(512 / RB), smem, stream, p);
+    hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, true, RB, KVLEN>), dim3((unsigned)p.st.G), dim3(512 / RB), smem, stream, p);
     PA_CHECK_LAUNCH("attention kernel (resident workgroups, bounded scores)");
   }
-  hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, false, RB>), dim3((unsigned)p.st.G), dim3(512 / RB), smem, stream, p);
+  hipLaunchKernelGGL((attn_fwd_d128_stream_kernel<T, false, RB, KVLEN>), dim3((unsigned)p.st.G), dim3(512 / RB), smem, stream, p);
   PA_CHECK_LAUNCH("attention kernel (resident workgroups)");
   return PA_OK;
 }
@@ -4055,7 +4115,9 @@ static int launch_stream(const AttnParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(clear_word_kernel, dim3(1), dim3(1), 0, stream, p.st.next_range, p.gate, p.gate_want);
     PA_CHECK_LAUNCH("range counter");
   }
-  const int rc = tuning().wave_rows == 64 ? launch_stream_rb<T, 2>(p, stream) : launch_stream_rb<T, 1>(p, stream);
+  // (per-batch key counts: the form with 32 rows per wavefront only)
+  const int rc = p.st.has_kvlen ? launch_stream_rb<T, 1, true>(p, stream)
+                 : tuning().wave_rows == 64 ? launch_stream_rb<T, 2, false>(p, stream) : launch_stream_rb<T, 1, false>(p, stream);
   if (rc != PA_OK) return rc;
   const int p_tail = p.st.n_pieces - p.st.R * p.st.G;
   if (p_tail > 0 && p.st.Gt != p_tail) {
@@ -4064,6 +4126,9 @@ static int launch_stream(const AttnParams& p, hipStream_t stream) {
   }
   return PA_OK;
 }
+
+// Where launch_bound leaves its flag in `ws`.
+static const int* bound_flag_address(const void* ws, int nseg) { return (const int*)((const float*)ws + (size_t)2 * BOUND_G * nseg); }
 
 // Launches the two small kernels that bound the scores (see score_bound_partial_kernel) into `ws` and returns the flag's address.
 static int launch_bound(const AttnParams& p, int dtype, int D, const KeySegs* segs, void* ws, hipStream_t st, const int** flag_out) {
@@ -4091,13 +4156,21 @@ static int launch_bound(const AttnParams& p, int dtype, int D, const KeySegs* se
   return PA_OK;
 }
 
+// Extras of a dense call that pa_attn_fwd_masked makes twice over one workspace, under a gate that lets one run.
+struct DenseOpts {
+  bool stream_kvlen = false;  // the per-batch key counts leave nearly all keys wherever the gate lets this call run: they may go
+                              // to the resident-workgroup kernel, and the call fails if that kernel does not take the shape
+  int* bound_done = nullptr;  // in/out: the score bound's words at the front of the workspace are (now) computed
+};
+
 static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out, float* lse,
                           int dtype, int B, int H, int Sq, int Skv, int D,
                           const int64_t q_strides[3], const int64_t k_strides[3],
                           const int64_t v_strides[3], const int64_t out_strides[3], float scale,
                           const int32_t* kv_len, int is_causal, void* workspace, size_t workspace_bytes,
                           void* stream, float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0,
-                          const int* gate = nullptr, int gate_want = 0, const KeySegs* segs = nullptr) {
+                          const int* gate = nullptr, int gate_want = 0, const KeySegs* segs = nullptr,
+                          const DenseOpts* opts = nullptr) {
   const int64_t zero3[3] = {0, 0, 0};
   const bool accumulate = acc_out != nullptr;
   if (accumulate) {
@@ -4124,7 +4197,10 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   const size_t bound_bytes = bound_ws_bytes(nseg);
   const bool want_bound = bound_wanted(B, H, Sq, Skv, D);
   size_t stream_bytes = 0;
-  bool streamed = plan_stream(p, D, segs, ws_avail > bound_bytes && want_bound ? ws_avail - bound_bytes : ws_avail, false, &stream_bytes);
+  const bool stream_kvlen = opts != nullptr && opts->stream_kvlen && !accumulate;
+  bool streamed = plan_stream(p, D, segs, ws_avail > bound_bytes && want_bound ? ws_avail - bound_bytes : ws_avail, false, &stream_bytes,
+                              true, stream_kvlen);
+  if (stream_kvlen && !streamed) PA_FAIL(PA_ERR_LAUNCH, "the resident-workgroup kernel does not take this shape (launch plans disagree)");
   if (!streamed) choose_kernel(p, D, 256, true, ws_avail, nullptr);
   if (segs && !streamed) {
     if (D != 128 || !p.pipe || p.causal || kv_len != nullptr || segs->n > MAX_KEY_SEGS ||
@@ -4142,8 +4218,13 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
                              : p.split_s > 1 ? (size_t)p.split_tiles * p.split_s * p.bm * (128 + 1) * sizeof(float) : 0;
   if (want_bound && p.pipe && (D == 64 || p.bm == 256) && ws_avail >= split_bytes + bound_bytes) {
     ws_base += bound_bytes;
-    rc = launch_bound(p, dtype, D, segs, workspace, (hipStream_t)stream, &p.bound_flag);
-    if (rc) return rc;
+    if (opts != nullptr && opts->bound_done != nullptr && *opts->bound_done) {
+      p.bound_flag = bound_flag_address(workspace, nseg);
+    } else {
+      rc = launch_bound(p, dtype, D, segs, workspace, (hipStream_t)stream, &p.bound_flag);
+      if (rc) return rc;
+      if (opts != nullptr && opts->bound_done != nullptr) *opts->bound_done = 1;
+    }
   }
   if (accumulate) {
     if (p.causal) PA_FAIL(PA_ERR_UNSUPPORTED, "ring accumulation is not causal");
@@ -4305,6 +4386,23 @@ static int launch_masked(const AttnParams& p, int mask_kind, hipStream_t stream)
   return PA_OK;
 }
 
+// Whether a dense call with per-batch key counts that leave nearly all keys would go to the resident-workgroup
+// kernel: where that kernel takes the shape with `ws_avail` bytes of workspace and the launch is a long one (from
+// 1024 key-tile steps per workgroup on, where its 7 % over the pipelined kernel outweigh a third, empty launch).
+static bool stream_takes_key_counts(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3], const int64_t v_strides[3], size_t ws_avail) {
+  if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D != 128) return false;
+  const int64_t zero[3] = {0, 0, 0};
+  static const int32_t some_count = 0;
+  AttnParams p;
+  fill_params(p, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, Sq, Skv, zero, k_strides, v_strides, zero, 1.f);
+  p.kv_len = &some_count;  // never read: only its presence counts for the plan
+  const size_t bound_bytes = bound_ws_bytes(1);
+  const bool want_bound = bound_wanted(B, H, Sq, Skv, D);
+  size_t need = 0;
+  if (!plan_stream(p, D, nullptr, ws_avail > bound_bytes && want_bound ? ws_avail - bound_bytes : ws_avail, false, &need, true, true)) return false;
+  return (int64_t)p.st.n_pieces * p.st.L >= (int64_t)1024 * p.st.G;
+}
+
 // Words at the front of pa_attn_fwd_masked's workspace: kept-key counts per batch element and the prefix flag.
 static size_t mask_scan_bytes(int B) { return (((size_t)B + 1) * sizeof(int32_t) + 255) & ~(size_t)255; }
 
@@ -4345,11 +4443,25 @@ extern "C" int pa_attn_fwd_masked(const void* q, const void* k, const void* v, v
   const size_t scan = mask_scan_bytes(B);
   if (key_only && any && workspace && workspace_bytes >= scan) {
     int32_t* words = (int32_t*)workspace;
-    hipLaunchKernelGGL(key_mask_scan_kernel, dim3(1), dim3(1024), 0, st, (const uint8_t*)mask, p.ms_b, p.ms_k, B, Skv, words);
+    // Long launches whose counts leave nearly all keys (a text prompt's padding at the end of 119k tokens) go to the
+    // resident-workgroup kernel, whose plan is made for all keys; the scan tells the two cases apart (flag 2 / 1)
+    // and a third launch is enqueued, of which again only one runs.  Both dense launches use the same workspace.
+    int bound_done = 0;
+    DenseOpts nearly_all, fewer;
+    nearly_all.stream_kvlen = true;
+    nearly_all.bound_done = fewer.bound_done = &bound_done;
+    const bool dual = stream_takes_key_counts(B, H, Sq, Skv, D, k_strides, v_strides, workspace_bytes - scan);
+    hipLaunchKernelGGL(key_mask_scan_kernel, dim3(1), dim3(1024), 0, st, (const uint8_t*)mask, p.ms_b, p.ms_k, B, Skv, words, dual ? 1 : 0);
     PA_CHECK_LAUNCH("key mask scan kernel");
+    if (dual) {
+      rc = attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
+                          scale, words, 0, (char*)workspace + scan, workspace_bytes - scan, stream, nullptr, nullptr, 0,
+                          words + B, 2, nullptr, &nearly_all);
+      if (rc) return rc;
+    }
     rc = attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
                         scale, words, 0, (char*)workspace + scan, workspace_bytes - scan, stream, nullptr, nullptr, 0,
-                        words + B, 1);
+                        words + B, 1, nullptr, &fewer);
     if (rc) return rc;
     p.gate = words + B;
     p.gate_want = 0;

@@ -298,6 +298,48 @@ def test_key_masks_take_the_fast_kernels_when_prefixes(cuda, tuning):
         assert torch.isfinite(lse).all()
 
 
+@pytest.mark.parametrize("rounds", [-1, 6])
+def test_long_launches_with_nearly_full_key_masks(cuda, rounds, tuning):
+    """A long launch (1024 key-tile steps per workgroup and more) whose key mask is a prefix that keeps at least 7/8 of
+    the keys in every batch element -- a padded text prompt at the end of a video's tokens -- goes to the
+    resident-workgroup kernel with the counts as per-batch key limits: pieces end at their batch element's last key,
+    ranges of the tail that lie beyond it come out empty (with 6 rounds the last ranges are 32 tiles long and one
+    batch element drops 60).  A prefix that keeps less goes to the kernel with one workgroup per query tile, anything
+    else to the per-score kernel; which of the three runs is decided on the device.  Sampled rows of three heads
+    against the fp64 oracle; the nearly full case also against the same call with the resident-workgroup kernel
+    switched off, and bit for bit against a second call."""
+    tuning("stream_dyn", rounds)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    B, H, D = 2, 8, 128
+    Sq, Skv = cus // 8 * 256 - 77, 64 * 520 + 13  # 2 x 8 x 32 pieces of 521 tiles: 1042 steps per workgroup
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=47)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    op = torch.ops.para_attn.attention_forward_with_lse
+    heads = [0, 3, 7]
+    rows = torch.cat([torch.arange(0, 150), torch.randint(0, Sq, (150,), generator=torch.Generator().manual_seed(2)), torch.arange(Sq - 150, Sq)])
+    cases = [("nearly full", [Skv - 3, Skv - 64 * 60 - 5]),  # the second batch element is the one whose pieces make up the tail ("full", [Skv, Skv]), ("nearly full, whole tiles", [Skv - 13, Skv - 13 - 128]),
+             ("half", [Skv - 3, Skv // 2]), ("scattered", None)]
+    for name, lens in cases:
+        if lens is None:
+            m = torch.arange(Skv)[None, :] < torch.tensor([Skv - 3, Skv - 70])[:, None]
+            m[1, 10] = False
+        else:
+            m = torch.arange(Skv)[None, :] < torch.tensor(lens)[:, None]
+        mask = m[:, None, None, :].to(cuda)
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, heads][:, :, rows].float().numpy(), k[:, heads].float().numpy(), v[:, heads].float().numpy(), None, m[:, None, None, :].numpy())
+        out, lse = op(qd, kd, vd, mask)
+        _check(out[:, heads][:, :, rows.to(cuda)], lse[:, heads][:, :, rows.to(cuda)], ref_out, ref_lse, f"{name}, rounds={rounds}")
+        assert torch.isfinite(lse).all() and torch.isfinite(out.float()).all()
+        out2, lse2 = op(qd, kd, vd, mask)
+        assert torch.equal(out2, out) and torch.equal(lse2, lse), name
+        if name.startswith("nearly"):
+            tuning("stream", 0)
+            out0, lse0 = op(qd, kd, vd, mask)
+            tuning("stream", -1)
+            assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
+            assert not torch.equal(out0, out), "meant to run two different kernels"
+
+
 @pytest.mark.parametrize("D", [128, 64])
 def test_empty_inputs(cuda, D):
     """No keys at all (Skv = 0, or a batch element whose mask keeps nothing): out = 0 and lse = -inf, what the
