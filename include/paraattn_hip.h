@@ -151,7 +151,9 @@ PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void*
  * A boolean mask that only selects keys (head and query strides 0: the text
  * padding masks of src/para_attn/ops/__init__.py:248-299) is scanned on the
  * device; where it keeps a prefix of the keys in every batch element the fast
- * dense kernels run with the counts as kv_len, otherwise, and for every other
+ * dense kernels run with the counts as kv_len (long launches whose prefixes
+ * keep at least 7/8 of the keys everywhere: the kernel with resident
+ * workgroups, which plain dense calls use), otherwise, and for every other
  * mask, a kernel that reads the mask per score.  The choice is made on the
  * device: nothing is read back, so the call can be captured in a HIP graph.
  * workspace: pa_attn_fwd_masked_workspace_bytes() bytes (16-byte aligned, any
