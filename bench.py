@@ -144,11 +144,13 @@ def bench_attn(dev, steps, warmup):
     return (q, k, v), 4.0 * B * H * S * S * D, t, checked
 
 
-def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=(0,), traffic=None, causal=False, sets=1):
+def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=(0,), traffic=None, causal=False, sets=1,
+                masked_keys=0):
     """One dense shape: timed, then sampled rows of the last timed output checked against torch's CPU SDPA.
     ``sets`` > 1: the calls rotate over that many copies of q, k, v at different addresses, so that a working set
     smaller than the 256 MB memory-side cache is not served from it call after call (in a model every call brings
-    other tensors)."""
+    other tensors).  ``masked_keys`` > 0: the call passes a boolean key mask [1,1,1,Skv] that drops that many keys
+    at the end (a padded text prompt); flops and the check are those of the kept keys."""
     import torch
 
     from oracle import inputs
@@ -157,21 +159,23 @@ def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=
     bufs = [(q.to(dev), k.to(dev), v.to(dev)) for _ in range(sets)]
     op = torch.ops.para_attn.attention_forward_with_lse
     last = {}
+    kept = Skv - masked_keys
+    mask = (torch.arange(Skv, device=dev) < kept)[None, None, None, :] if masked_keys else None
 
     def call(i):
         qd, kd, vd = bufs[i % sets]
-        last["out"], last["lse"] = op(qd, kd, vd, is_causal=causal)
+        last["out"], last["lse"] = op(qd, kd, vd, mask, is_causal=causal)
 
     t = _time_calls(call, steps, warmup)
     heads = sorted(set(list(check_heads) + [H - 1]))
-    checked = _check_rows(last["out"], last["lse"], q, k, v, heads, _sample_rows(Sq), name, causal=causal)
-    flops = 4.0 * B * H * Sq * Skv * D * (0.5 if causal else 1.0)  # causal: the kept half (Sq == Skv)
+    checked = _check_rows(last["out"], last["lse"], q, k[:, :, :kept], v[:, :, :kept], heads, _sample_rows(Sq), name, causal=causal)
+    flops = 4.0 * B * H * Sq * kept * D * (0.5 if causal else 1.0)  # causal: the kept half (Sq == Skv)
     nbytes = 2.0 * B * H * D * (2 * Sq + 2 * Skv) + 4.0 * B * H * Sq
     gbs = nbytes / (t["median"] * 1e-3) / 1e9
     more = {"traffic": TRAFFIC[traffic], "traffic_source": TRAFFIC_SOURCE} if traffic else {}
     if sets > 1:
         more["buffer_sets"] = sets
-    what = "attention_forward_with_lse" + (" is_causal" if causal else "")
+    what = "attention_forward_with_lse" + (" is_causal" if causal else "") + (f" with a key mask that drops the last {masked_keys} keys" if masked_keys else "")
     return _mfma(f"{name}: {what} q [{B},{H},{Sq},{D}] k,v [{B},{H},{Skv},{D}] bf16", flops, t,
                  bytes=nbytes, gbs=round(gbs, 1), frac_hbm=round(gbs / PEAK_HBM_GBS, 4), checked=checked, **more)
 
@@ -227,10 +231,13 @@ def bench_ring(dev, steps=6, warmup=3):
 
 
 def bench_shapes(dev, steps=10, warmup=5):
-    """Two further dense shapes: the headline shape with is_causal (flops of the kept half) and a head_dim 64 shape."""
+    """Further dense shapes: the headline shape with is_causal (flops of the kept half), the headline shape with the
+    key mask of a padded text prompt, and a head_dim 64 shape."""
     return {
         "headline_shape_causal": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=5,
                                              check_heads=(0, 1), causal=True, traffic="causal"),
+        "headline_shape_text_mask": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=7,
+                                                check_heads=(0, 1), masked_keys=167),
         "head_dim_64": _dense_case(dev, "head_dim 64 (CogVideoX-like)", 1, 48, 17776, 17776, 64, steps, warmup, seed=6,
                                    check_heads=(0, 23), traffic="head_dim_64"),
     }
@@ -503,7 +510,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "pa::attn_fwd_d128_stream_kernel<pa::BF16, true, 1>",
+            "kernel": "pa::attn_fwd_d128_stream_kernel<pa::BF16, true, 1, false>",
             "achieved": round(kern_tflops, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
