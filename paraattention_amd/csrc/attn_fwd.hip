@@ -4387,8 +4387,10 @@ static int launch_masked(const AttnParams& p, int mask_kind, hipStream_t stream)
 }
 
 // Whether a dense call with per-batch key counts that leave nearly all keys would go to the resident-workgroup
-// kernel: where that kernel takes the shape with `ws_avail` bytes of workspace and the launch is a long one (from
-// 1024 key-tile steps per workgroup on, where its 7 % over the pipelined kernel outweigh a third, empty launch).
+// kernel: where that kernel takes the shape with `ws_avail` bytes of workspace and the launch is long enough for its
+// advantage over the kernel with one workgroup per query tile to outweigh a third, empty launch: from 512 key-tile
+// steps per workgroup on (measured with 100 keys masked: +5 / +1 % at 121 / 216 steps, level at 384, -0.7 .. -1 % at
+// 576 .. 640, -2 .. -3 % from 1536 on, -5 % at the 119k-token shape).
 static bool stream_takes_key_counts(int B, int H, int Sq, int Skv, int D, const int64_t k_strides[3], const int64_t v_strides[3], size_t ws_avail) {
   if (B <= 0 || H <= 0 || Sq <= 0 || Skv <= 0 || D != 128) return false;
   const int64_t zero[3] = {0, 0, 0};
@@ -4400,7 +4402,7 @@ static bool stream_takes_key_counts(int B, int H, int Sq, int Skv, int D, const 
   const bool want_bound = bound_wanted(B, H, Sq, Skv, D);
   size_t need = 0;
   if (!plan_stream(p, D, nullptr, ws_avail > bound_bytes && want_bound ? ws_avail - bound_bytes : ws_avail, false, &need, true, true)) return false;
-  return (int64_t)p.st.n_pieces * p.st.L >= (int64_t)1024 * p.st.G;
+  return (int64_t)p.st.n_pieces * p.st.L >= (int64_t)512 * p.st.G;
 }
 
 // Words at the front of pa_attn_fwd_masked's workspace: kept-key counts per batch element and the prefix flag.
@@ -4443,7 +4445,7 @@ extern "C" int pa_attn_fwd_masked(const void* q, const void* k, const void* v, v
   const size_t scan = mask_scan_bytes(B);
   if (key_only && any && workspace && workspace_bytes >= scan) {
     int32_t* words = (int32_t*)workspace;
-    // Long launches whose counts leave nearly all keys (a text prompt's padding at the end of 119k tokens) go to the
+    // Longer launches whose counts leave nearly all keys (a text prompt's padding at the end of 119k tokens) go to the
     // resident-workgroup kernel, whose plan is made for all keys; the scan tells the two cases apart (flag 2 / 1)
     // and a third launch is enqueued, of which again only one runs.  Both dense launches use the same workspace.
     int bound_done = 0;

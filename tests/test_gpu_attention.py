@@ -300,7 +300,7 @@ def test_key_masks_take_the_fast_kernels_when_prefixes(cuda, tuning):
 
 @pytest.mark.parametrize("rounds", [-1, 6])
 def test_long_launches_with_nearly_full_key_masks(cuda, rounds, tuning):
-    """A long launch (1024 key-tile steps per workgroup and more) whose key mask is a prefix that keeps at least 7/8 of
+    """A longer launch (512 key-tile steps per workgroup and more) whose key mask is a prefix that keeps at least 7/8 of
     the keys in every batch element -- a padded text prompt at the end of a video's tokens -- goes to the
     resident-workgroup kernel with the counts as per-batch key limits: pieces end at their batch element's last key,
     ranges of the tail that lie beyond it come out empty (with 6 rounds the last ranges are 32 tiles long and one
