@@ -38,9 +38,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # Traffic at the L2's memory side per launch in bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two
 # rocprofv3 --pmc runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy).  These counters cannot be
 # read from inside this process; the figures are those of the summary named in TRAFFIC_SOURCE, not of this run.
-TRAFFIC = {"attn": 1.006e10, "merge": 4.771e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 9.250e9,
-           "flux": 3.017e8, "ring_sweep": 1.234e10, "ring_sweep_per_block": 1.436e10, "wan_self": 3.745e9, "wan_cross": 7.018e8,
-           "causal": 5.160e9, "head_dim_64": 2.438e9}
+TRAFFIC = {"attn": 1.005e10, "merge": 4.773e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 8.940e9,
+           "flux": 3.039e8, "ring_sweep": 1.234e10, "ring_sweep_per_block": 1.436e10, "wan_self": 3.797e9, "wan_cross": 7.013e8,
+           "causal": 5.153e9, "text_mask": 1.005e10, "head_dim_64": 2.438e9}
 TRAFFIC_SOURCE = "profiles/kernels_bench_workloads.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the same command)"
 
 
@@ -237,7 +237,7 @@ def bench_shapes(dev, steps=10, warmup=5):
         "headline_shape_causal": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=5,
                                              check_heads=(0, 1), causal=True, traffic="causal"),
         "headline_shape_text_mask": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=7,
-                                                check_heads=(0, 1), masked_keys=167),
+                                                check_heads=(0, 1), masked_keys=167, traffic="text_mask"),
         "head_dim_64": _dense_case(dev, "head_dim 64 (CogVideoX-like)", 1, 48, 17776, 17776, 64, steps, warmup, seed=6,
                                    check_heads=(0, 23), traffic="head_dim_64"),
     }
