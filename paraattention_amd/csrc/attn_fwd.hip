@@ -2024,8 +2024,9 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
       int* const counter = kp->st.next_range;
       int n;
       if (counter != nullptr) {
-        // Every wavefront of the workgroup comes by here in the same iteration.  Wavefront 0 draws the number; the
-        // word it leaves in LDS is not written again before the next draw, at least 16 barriers later.
+        // Every wavefront of the workgroup comes by here in the same iteration.  Wavefront 0 draws the number and
+        // leaves it in LDS; the second barrier keeps it from writing the next one (an empty range is followed by
+        // another draw at once) before every wavefront has read this one.
         if (wave == 0) {
           int v = 0;
           if (lane == 0) v = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -2033,6 +2034,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
         }
         __syncthreads();
         n = __builtin_amdgcn_readfirstlane(*(volatile int*)sTaken);
+        __syncthreads();
         if (n < 0) return false;
       } else if (!g_in_tail) {
         n = wg;
