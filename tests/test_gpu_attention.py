@@ -556,6 +556,47 @@ def test_one_workgroup_draws_every_range(cuda, rounds, wave_rows, tuning):
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
 
 
+def test_drawn_ranges_random_configurations(cuda, tuning):
+    """Sixteen seeded random draws for the resident-workgroup kernel with drawn tail ranges forced on: batch, heads,
+    query rows and keys such that the work is 300 to 1200 key-tile steps per workgroup (whole rounds of pieces or
+    none, tails of every size), 2 to 6 rounds, either dtype, [B,H,S,D] or [B,S,H,D] memory, and in half of the cases a
+    prefix key mask that keeps at least 7/8 of the keys of every batch element (the variant with per-batch key counts
+    where the launch is long enough for it, the kernel with one workgroup per query tile below).  Sampled rows of up
+    to three heads against the fp64 oracle, and the same bits from a second call."""
+    tuning("stream", 1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rng = np.random.default_rng(2024)
+    op = torch.ops.para_attn.attention_forward_with_lse
+    for case in range(16):
+        B, H = int(rng.integers(1, 3)), int(rng.integers(1, 7))
+        steps = int(rng.integers(300, 1200)) * cus          # key-tile steps of the whole launch
+        L = int(rng.integers(40, 700))                       # key tiles per piece
+        pieces = max(B * H, steps // L)
+        Sq = max(1, pieces // (B * H)) * 256 - int(rng.integers(0, 256))
+        Skv = L * 64 - int(rng.integers(0, 64))
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+        tuning("stream_dyn", int(rng.integers(2, 7)))
+        q, k, v = inputs.qkv(B, H, Sq, Skv, 128, seed=4000 + case, dtype=dtype)
+        keep = None
+        if case % 2:
+            lens = [int(rng.integers(Skv - Skv // 8, Skv + 1)) for _ in range(B)]
+            keep = torch.arange(Skv)[None, :] < torch.tensor(lens)[:, None]
+        heads = sorted(set([0, H // 2, H - 1]))
+        rows = torch.cat([torch.arange(0, min(Sq, 120)), torch.randint(0, Sq, (120,), generator=torch.Generator().manual_seed(case)), torch.arange(max(0, Sq - 120), Sq)])
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, heads][:, :, rows].float().numpy(), k[:, heads].float().numpy(), v[:, heads].float().numpy(),
+                                              None, None if keep is None else keep[:, None, None, :].numpy())
+        dev = [t.to(cuda) for t in (q, k, v)]
+        for i in range(3):
+            if rng.random() < 0.4:
+                dev[i] = dev[i].transpose(1, 2).contiguous().transpose(1, 2)
+        mask = None if keep is None else keep[:, None, None, :].to(cuda)
+        out, lse = op(*dev, mask)
+        what = f"case {case}: B{B} H{H} Sq{Sq} Skv{Skv} {dtype} masked={keep is not None}"
+        _check(out[:, heads][:, :, rows.to(cuda)], lse[:, heads][:, :, rows.to(cuda)], ref_out, ref_lse, what)
+        out2, lse2 = op(*dev, mask)
+        assert torch.equal(out2, out) and torch.equal(lse2, lse), what
+
+
 def test_planner_draws_ranges_for_long_launches_only(cuda, tuning):
     """What the planner asks of the workspace says which plan it took: four rounds of ranges (4 x compute units x two
     partial results, and the counter's 256 bytes) from 1024 key-tile steps per workgroup on, at most one range per
