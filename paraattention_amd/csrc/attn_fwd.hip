@@ -125,12 +125,15 @@ struct AttnParams {
   // MASK_F32 / MASK_ACT: a bias added to the scaled score (fp32, or the activation type).
   const void* mask;
   int64_t ms_b, ms_h, ms_q, ms_k;
-  // dense kernels: with `gate` set the launch leaves at once unless *gate == gate_want (a decision taken on
+  // dense kernels: with `gate` set the launch leaves at once unless bit *gate of gate_mask is set (a decision taken on
   // the device by an earlier launch of the same stream, e.g. whether a key mask is a prefix)
   const int* gate;
-  int gate_want;
+  uint32_t gate_mask;
   StreamPlan st;  // attn_fwd_d128_stream_kernel only
 };
+
+// Whether the value that an earlier launch left in *gate (0 .. 31) is one of those a launch runs for.
+__device__ __forceinline__ bool gate_open(const int* gate, uint32_t mask) { return ((mask >> (*gate & 31)) & 1u) != 0; }
 
 constexpr int MASK_NONE = 0, MASK_BOOL = 1, MASK_F32 = 2, MASK_ACT = 3;
 
@@ -268,7 +271,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
   typedef typename T::vec8 vec8;
   typedef Smem<D> SM;
   if constexpr (!SPARSE) {
-    if (p.gate != nullptr && *p.gate != p.gate_want) return;
+    if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   }
   constexpr int DC = D / 16;   // contraction chunks of the first GEMM
   constexpr int DB = D / 32;   // 32-row blocks of O^T
@@ -599,7 +602,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_d128_kernel(const AttnPa
   typedef typename T::vec8 vec8;
   constexpr int D = 128, DC = 8, DB = 4;
   if constexpr (!SPARSE) {
-    if (p.gate != nullptr && *p.gate != p.gate_want) return;
+    if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   }
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                    // [2][64][256 B]
@@ -945,7 +948,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d128_pipe_k
     if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
   }
   if constexpr (!SPARSE) {
-    if (p.gate != nullptr && *p.gate != p.gate_want) return;
+    if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   }
   constexpr int RS = 4 * NW;    // tile rows between two of them
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
@@ -1491,7 +1494,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_fwd_d64_pipe_ke
   // BOUNDED and the flag: as in attn_fwd_d128_pipe_kernel
   if constexpr (!SPARSE) {
     if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
-    if (p.gate != nullptr && *p.gate != p.gate_want) return;
+    if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   }
   typedef typename T::vec8 vec8;
   constexpr int DC = 4, DB = 2;
@@ -1887,7 +1890,7 @@ __global__ __launch_bounds__(512 / RB, 1) void attn_fwd_d128_stream_kernel(const
   constexpr int IPW = 16 / NW;  // copy instructions per wavefront and K (V) tile
   constexpr int RS = 4 * NW;    // tile rows between two of them
   if (p.bound_flag != nullptr && (*p.bound_flag != 0) != BOUNDED) return;
-  if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                    // [2][64][256 B]
   char* const sV = (char*)smem + 2 * TILE_BYTES;   // [2][64][256 B]
@@ -2726,7 +2729,7 @@ template <typename T>
 __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnParams p) {
   typedef typename T::vec8 vec8;
   constexpr int DC = 8, DB = 4, NT = SHORT_NT, QI = SHORT_QI;
-  if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   char* const sK = (char*)smem;                   // [2][64][256 B]
   char* const sV = (char*)smem + 2 * TILE_BYTES;  // [2][64][256 B]
@@ -3140,7 +3143,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_d128_short_kernel(const AttnP
 // ring accumulation.  16 workgroups per tail piece, 16 query rows each; one thread = 8 consecutive output elements.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_stream_merge_kernel(const AttnParams p) {
-  if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   const StreamPlan& sp = p.st;
   const int tp = blockIdx.x >> 4;  // tail piece
   const int local = ((blockIdx.x & 15) << 4) + (threadIdx.x >> 4);
@@ -3208,7 +3211,7 @@ __global__ __launch_bounds__(256) void attn_stream_merge_kernel(const AttnParams
 // once.  One thread = 8 consecutive output elements of one query row; 16 rows per workgroup.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_split_merge_kernel(const AttnParams p) {
-  if (p.gate != nullptr && *p.gate != p.gate_want) return;
+  if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
   const int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int c8 = (threadIdx.x & 15) * 8;
   const int tl = (int)(r / p.bm), local = (int)(r % p.bm);
@@ -3510,8 +3513,11 @@ __global__ __launch_bounds__(256) void score_bound_flag_kernel(const float* part
 // whether in every batch element the kept keys are exactly the leading ones (then the dense kernels take the
 // counts as kv_len and the mask need not be looked at again).  One workgroup; out[0..B) = counts,
 // out[B] = 1 if all are prefixes else 0.
-__global__ __launch_bounds__(1024) void key_mask_scan_kernel(const uint8_t* mask, int64_t mb, int64_t mk, int B,
-                                                             int Skv, int32_t* out, int tell_nearly_all) {
+// A boolean key mask is taken apart on the device.  Result: out[b] = kept keys of batch element b; out[B] = bit 0:
+// every element keeps a prefix of its keys, bit 1: every element keeps at least 7/8 of them.
+// Short masks: one workgroup does it all.
+__global__ __launch_bounds__(1024) void key_mask_small_kernel(const uint8_t* mask, int64_t mb, int64_t mk, int B,
+                                                              int Skv, int32_t* out) {
   __shared__ int s_cnt[1024];
   __shared__ int s_last[1024];
   int all_prefix = 1, fewest = Skv;
@@ -3538,8 +3544,131 @@ __global__ __launch_bounds__(1024) void key_mask_scan_kernel(const uint8_t* mask
     fewest = min(fewest, s_cnt[0]);
     __syncthreads();
   }
-  // 0: not prefixes; 1: prefixes; 2 (where asked for): prefixes that keep at least 7/8 of the keys in every batch element
-  if (threadIdx.x == 0) out[B] = !all_prefix ? 0 : tell_nearly_all && (int64_t)fewest * 8 >= (int64_t)Skv * 7 ? 2 : 1;
+  if (threadIdx.x == 0) out[B] = all_prefix | ((int64_t)fewest * 8 >= (int64_t)Skv * 7 ? 2 : 0);
+}
+
+// Long masks, first step: kept keys and last kept key of every chunk of MASK_CHUNK keys (one workgroup per chunk
+// and batch element).
+constexpr int MASK_CHUNK = 1024;
+__global__ __launch_bounds__(256) void key_mask_chunk_kernel(const uint8_t* mask, int64_t mb, int64_t mk, int Skv, int nchunk,
+                                                             int32_t* chunk_cnt, int32_t* chunk_last) {
+  __shared__ int s_cnt[256];
+  __shared__ int s_last[256];
+  const int b = blockIdx.y, c = blockIdx.x, t = threadIdx.x;
+  const uint8_t* mrow = mask + (int64_t)b * mb;
+  int cnt = 0, last = -1;
+  for (int i = 0; i < MASK_CHUNK / 256; ++i) {
+    const int j = c * MASK_CHUNK + i * 256 + t;
+    if (j < Skv && mrow[(int64_t)j * mk] != 0) {
+      ++cnt;
+      last = j;
+    }
+  }
+  s_cnt[t] = cnt;
+  s_last[t] = last;
+  __syncthreads();
+  for (int d = 128; d > 0; d >>= 1) {
+    if (t < d) {
+      s_cnt[t] += s_cnt[t + d];
+      s_last[t] = max(s_last[t], s_last[t + d]);
+    }
+    __syncthreads();
+  }
+  if (t == 0) {
+    chunk_cnt[b * nchunk + c] = s_cnt[0];
+    chunk_last[b * nchunk + c] = s_last[0];
+  }
+}
+
+// Second step (one workgroup): where each chunk's kept keys begin among its batch element's kept keys, and the result.
+__global__ __launch_bounds__(256) void key_mask_scan_kernel(int B, int Skv, int nchunk, const int32_t* chunk_cnt, const int32_t* chunk_last,
+                                                            int32_t* chunk_off, int32_t* out) {
+  __shared__ int s_scan[256];
+  __shared__ int s_last[256];
+  const int t = threadIdx.x;
+  int all_prefix = 1, fewest = Skv;
+  for (int b = 0; b < B; ++b) {
+    int running = 0, last = -1;
+    for (int base = 0; base < nchunk; base += 256) {
+      const int c = base + t;
+      const int v = c < nchunk ? chunk_cnt[b * nchunk + c] : 0;
+      s_scan[t] = v;
+      s_last[t] = c < nchunk ? chunk_last[b * nchunk + c] : -1;
+      __syncthreads();
+      for (int d = 1; d < 256; d <<= 1) {
+        const int add = t >= d ? s_scan[t - d] : 0;
+        const int other = t >= d ? s_last[t - d] : -1;
+        __syncthreads();
+        s_scan[t] += add;
+        s_last[t] = max(s_last[t], other);
+        __syncthreads();
+      }
+      if (c < nchunk) chunk_off[b * nchunk + c] = running + s_scan[t] - v;
+      running += s_scan[255];
+      last = max(last, s_last[255]);
+      __syncthreads();
+    }
+    if (t == 0) out[b] = running;
+    if (running != last + 1) all_prefix = 0;
+    fewest = min(fewest, running);
+  }
+  if (t == 0) out[B] = all_prefix | ((int64_t)fewest * 8 >= (int64_t)Skv * 7 ? 2 : 0);
+}
+
+// Gathers the kept key and value rows of a key mask that is not a prefix into dense copies [B][H][Skv][D] (the
+// reference's attention_forward_sparse_kv selects them with index_select, src/para_attn/ops/__init__.py:283-287), in
+// their order.  One workgroup per chunk of MASK_CHUNK keys, head and batch element: it ranks the chunk's kept keys
+// (wavefront ballots), then copies their rows to where the chunk's keys begin (chunk_off), 16 bytes per thread.  The
+// rows from the last kept key to the end of its key tile are cleared: the kernels read whole tiles, and a
+// probability of 0 times whatever the workspace held would still be a NaN.
+template <int D>
+__global__ __launch_bounds__(256) void gather_kept_keys_kernel(const AttnParams p, const uint8_t* mask, int64_t mb, int64_t mk, int nchunk,
+                                                               const int32_t* count, const int32_t* chunk_off, uint16_t* kc, uint16_t* vc) {
+  if (p.gate != nullptr && !gate_open(p.gate, p.gate_mask)) return;
+  constexpr int CPR = D / 8;      // 16-byte chunks per row
+  constexpr int RPB = 256 / CPR;  // rows per pass of the workgroup
+  __shared__ int s_src[MASK_CHUNK];
+  __shared__ int s_wave[4];
+  const int b = blockIdx.z, h = blockIdx.y, c = blockIdx.x, t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const uint8_t* mrow = mask + (int64_t)b * mb;
+  int m = 0;
+  for (int i = 0; i < MASK_CHUNK / 256; ++i) {
+    const int j = c * MASK_CHUNK + i * 256 + t;
+    const bool kept = j < p.Skv && mrow[(int64_t)j * mk] != 0;
+    const uint64_t votes = __ballot(kept);
+    if (lane == 0) s_wave[wave] = __popcll(votes);
+    __syncthreads();
+    int before = 0, all = 0;
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) before += s_wave[w];
+      all += s_wave[w];
+    }
+    if (kept) s_src[m + before + __popcll(votes & ((1ull << lane) - 1ull))] = j;
+    m += all;
+    __syncthreads();
+  }
+  const uint16_t* kb = (const uint16_t*)p.k + b * p.ks_b + h * p.ks_h;
+  const uint16_t* vb = (const uint16_t*)p.v + b * p.vs_b + h * p.vs_h;
+  const int64_t dst0 = ((int64_t)b * p.H + h) * p.Skv;
+  const int cc = t % CPR;
+  const int first = chunk_off[b * nchunk + c];
+  for (int r = t / CPR; r < m; r += RPB) {
+    const int64_t s_row = s_src[r];
+    const u32x4 kx = *(const u32x4*)(kb + s_row * p.ks_s + 8 * cc);
+    const u32x4 vx = *(const u32x4*)(vb + s_row * p.vs_s + 8 * cc);
+    *(u32x4*)(kc + (dst0 + first + r) * D + 8 * cc) = kx;
+    *(u32x4*)(vc + (dst0 + first + r) * D + 8 * cc) = vx;
+  }
+  if (c == nchunk - 1) {
+    const int n = count[b];
+    const int n_end = min(p.Skv, (n + BN - 1) / BN * BN);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int i = n + t / CPR; i < n_end; i += RPB) {
+      *(u32x4*)(kc + (dst0 + i) * D + 8 * cc) = z;
+      *(u32x4*)(vc + (dst0 + i) * D + 8 * cc) = z;
+    }
+  }
 }
 
 }  // namespace pa
@@ -3593,7 +3722,7 @@ static void fill_params(AttnParams& p, const void* q, const void* k, const void*
   p.split_main = 0; p.split_tiles = 0; p.split_s = 0; p.ws_out = nullptr; p.ws_lse = nullptr;
   p.bound_flag = nullptr;
   p.mask = nullptr; p.ms_b = p.ms_h = p.ms_q = p.ms_k = 0;
-  p.gate = nullptr; p.gate_want = 0;
+  p.gate = nullptr; p.gate_mask = 0;
   p.st = StreamPlan{};
 }
 
@@ -4105,8 +4234,8 @@ static int launch_stream_rb(const AttnParams& p, hipStream_t stream) {
   return PA_OK;
 }
 
-__global__ void clear_word_kernel(int* w, const int* gate, int gate_want) {
-  if (gate != nullptr && *gate != gate_want) return;
+__global__ void clear_word_kernel(int* w, const int* gate, uint32_t gate_mask) {
+  if (gate != nullptr && !gate_open(gate, gate_mask)) return;
   *w = 0;
 }
 
@@ -4114,7 +4243,7 @@ template <typename T>
 static int launch_stream(const AttnParams& p, hipStream_t stream) {
   if (p.out == nullptr && p.acc_out == nullptr) PA_FAIL(PA_ERR_INVALID, "null output pointer");
   if (p.st.next_range != nullptr) {  // a kernel, not a memset: the call may be under graph capture
-    hipLaunchKernelGGL(clear_word_kernel, dim3(1), dim3(1), 0, stream, p.st.next_range, p.gate, p.gate_want);
+    hipLaunchKernelGGL(clear_word_kernel, dim3(1), dim3(1), 0, stream, p.st.next_range, p.gate, p.gate_mask);
     PA_CHECK_LAUNCH("range counter");
   }
   // (per-batch key counts: the form with 32 rows per wavefront only)
@@ -4171,7 +4300,7 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
                           const int64_t v_strides[3], const int64_t out_strides[3], float scale,
                           const int32_t* kv_len, int is_causal, void* workspace, size_t workspace_bytes,
                           void* stream, float* acc_out = nullptr, float* acc_lse = nullptr, int acc_first = 0,
-                          const int* gate = nullptr, int gate_want = 0, const KeySegs* segs = nullptr,
+                          const int* gate = nullptr, uint32_t gate_mask = 0, const KeySegs* segs = nullptr,
                           const DenseOpts* opts = nullptr) {
   const int64_t zero3[3] = {0, 0, 0};
   const bool accumulate = acc_out != nullptr;
@@ -4189,7 +4318,7 @@ static int attn_fwd_dense(const void* q, const void* k, const void* v, void* out
   p.kv_len = kv_len;
   p.causal = is_causal != 0;
   p.gate = gate;
-  p.gate_want = gate_want;
+  p.gate_mask = gate_mask;
   if (!accumulate && !segs && plan_short(p, D))
     return dtype == PA_DTYPE_BF16 ? launch_short<BF16>(p, (hipStream_t)stream) : launch_short<F16>(p, (hipStream_t)stream);
   const size_t ws_avail = workspace ? workspace_bytes : 0;
@@ -4407,13 +4536,38 @@ static bool stream_takes_key_counts(int B, int H, int Sq, int Skv, int D, const 
   return (int64_t)p.st.n_pieces * p.st.L >= (int64_t)512 * p.st.G;
 }
 
-// Words at the front of pa_attn_fwd_masked's workspace: kept-key counts per batch element and the prefix flag.
-static size_t mask_scan_bytes(int B) { return (((size_t)B + 1) * sizeof(int32_t) + 255) & ~(size_t)255; }
+// Words at the front of pa_attn_fwd_masked's workspace: kept-key counts per batch element and the flag, then three
+// words per batch element and chunk of MASK_CHUNK keys (kept keys, last kept key, first position among the kept).
+static int mask_chunks(int Skv) { return (Skv + MASK_CHUNK - 1) / MASK_CHUNK; }
+static size_t mask_scan_bytes(int B, int Skv) {
+  return (((size_t)B + 1 + (size_t)3 * B * mask_chunks(Skv)) * sizeof(int32_t) + 255) & ~(size_t)255;
+}
+
+// pa_attn_fwd_masked's workspace when it gathers the kept keys of a mask with holes: the scan's words, dense copies
+// of K and V [B][H][Skv][D], then the workspace of the dense launches.
+struct MaskedLayout {
+  size_t kc, vc, dense;
+};
+static MaskedLayout masked_layout(int B, int H, int Skv, int D) {
+  auto up = [](size_t n) { return (n + 255) & ~(size_t)255; };
+  MaskedLayout l;
+  l.kc = mask_scan_bytes(B, Skv);
+  l.vc = l.kc + up((size_t)B * H * Skv * D * 2);
+  l.dense = l.vc + up((size_t)B * H * Skv * D * 2);
+  return l;
+}
 
 extern "C" size_t pa_attn_fwd_masked_workspace_bytes(int B, int H, int Sq, int Skv, int D,
                                                      const int64_t k_strides[3], const int64_t v_strides[3]) {
   if (B <= 0) return 0;
-  return mask_scan_bytes(B) + pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, k_strides, v_strides);
+  const size_t dense = pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, k_strides, v_strides);
+  if (H <= 0 || Sq <= 0 || Skv <= 0 || (D != 128 && D != 64)) return mask_scan_bytes(B, Skv > 0 ? Skv : 1) + dense;
+  // room to gather the kept keys of a mask with holes (from 3e11 flop on; see pa_attn_fwd_masked), and for the dense
+  // launches over the gathered copies, whose strides are those of contiguous tensors
+  if (4.0 * B * H * (double)Sq * (double)Skv * D < 3.0e11) return mask_scan_bytes(B, Skv > 0 ? Skv : 1) + dense;
+  const int64_t cs[3] = {(int64_t)H * Skv * D, (int64_t)Skv * D, D};
+  const size_t dense_c = pa_attn_fwd_workspace_bytes(B, H, Sq, Skv, D, cs, cs);
+  return masked_layout(B, H, Skv, D).dense + (dense > dense_c ? dense : dense_c);
 }
 
 extern "C" int pa_attn_fwd_masked(const void* q, const void* k, const void* v, void* out, float* lse,
@@ -4444,31 +4598,78 @@ extern "C" int pa_attn_fwd_masked(const void* q, const void* k, const void* v, v
   // small scan writes the kept-key counts and a flag, then both the dense launch (counts as kv_len) and the
   // masked launch are enqueued, and the one the flag does not select leaves at once.  Nothing is read back.
   const bool key_only = mask_kind == MASK_BOOL && (H == 1 || p.ms_h == 0) && (Sq == 1 || p.ms_q == 0);
-  const size_t scan = mask_scan_bytes(B);
+  const size_t scan = mask_scan_bytes(B, Skv > 0 ? Skv : 1);
   if (key_only && any && workspace && workspace_bytes >= scan) {
     int32_t* words = (int32_t*)workspace;
-    // Longer launches whose counts leave nearly all keys (a text prompt's padding at the end of 119k tokens) go to the
-    // resident-workgroup kernel, whose plan is made for all keys; the scan tells the two cases apart (flag 2 / 1)
-    // and a third launch is enqueued, of which again only one runs.  Both dense launches use the same workspace.
+    const int* flag = words + B;  // bit 0: prefixes; bit 1: at least 7/8 of the keys kept everywhere
+    constexpr uint32_t PREFIX_FEWER = 1u << 1, PREFIX_MOST = 1u << 3, HOLES_FEWER = 1u << 0, HOLES_MOST = 1u << 2;
+    // A mask with holes (what the reference's sequence-parallel HunyuanVideo adapter builds: every rank's text
+    // padding ends up inside the gathered sequence, context_parallel/diffusers_adapters/hunyuan_video.py:86-100) is
+    // served as the reference's attention_forward_sparse_kv serves it (ops/__init__.py:276-296): the kept K and V
+    // rows are gathered into dense copies, on which the fast kernels run with the counts as kv_len.  From 3e11 flop
+    // on (0.3 ms), where a handful of launches that return at once no longer count, and where the workspace has room.
+    const MaskedLayout lay = masked_layout(B, H, Skv, D);
+    const double flops = 4.0 * B * H * (double)Sq * (double)Skv * D;
+    const bool gather = flops >= 3.0e11 && workspace_bytes >= lay.dense;
+    const size_t dense_off = gather ? lay.dense : scan;
+    char* const dense_ws = (char*)workspace + dense_off;
+    const size_t dense_bytes = workspace_bytes - dense_off;
+    const int nchunk = mask_chunks(Skv);
+    int32_t* const chunk_cnt = words + B + 1;
+    int32_t* const chunk_last = chunk_cnt + (size_t)B * nchunk;
+    int32_t* const chunk_off = chunk_last + (size_t)B * nchunk;
+    if (gather || Skv > 8192) {
+      hipLaunchKernelGGL(key_mask_chunk_kernel, dim3(nchunk, B), dim3(256), 0, st, (const uint8_t*)mask, p.ms_b, p.ms_k, Skv, nchunk, chunk_cnt, chunk_last);
+      PA_CHECK_LAUNCH("key mask chunk kernel");
+      hipLaunchKernelGGL(key_mask_scan_kernel, dim3(1), dim3(256), 0, st, B, Skv, nchunk, (const int32_t*)chunk_cnt, (const int32_t*)chunk_last, chunk_off, words);
+      PA_CHECK_LAUNCH("key mask scan kernel");
+    } else {
+      hipLaunchKernelGGL(key_mask_small_kernel, dim3(1), dim3(1024), 0, st, (const uint8_t*)mask, p.ms_b, p.ms_k, B, Skv, words);
+      PA_CHECK_LAUNCH("key mask kernel");
+    }
     int bound_done = 0;
-    DenseOpts nearly_all, fewer;
-    nearly_all.stream_kvlen = true;
-    nearly_all.bound_done = fewer.bound_done = &bound_done;
-    const bool dual = stream_takes_key_counts(B, H, Sq, Skv, D, k_strides, v_strides, workspace_bytes - scan);
-    hipLaunchKernelGGL(key_mask_scan_kernel, dim3(1), dim3(1024), 0, st, (const uint8_t*)mask, p.ms_b, p.ms_k, B, Skv, words, dual ? 1 : 0);
-    PA_CHECK_LAUNCH("key mask scan kernel");
+    DenseOpts most, fewer;
+    most.stream_kvlen = true;
+    most.bound_done = fewer.bound_done = &bound_done;
+    // Longer launches whose counts leave nearly all keys (a text prompt's padding in 119k tokens) go to the
+    // resident-workgroup kernel, whose plan is made for all keys: one more launch, of which again only one runs.
+    // All dense launches of the call share one workspace and one score bound (computed over all keys).
+    bool dual = stream_takes_key_counts(B, H, Sq, Skv, D, k_strides, v_strides, dense_bytes);
     if (dual) {
       rc = attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
-                          scale, words, 0, (char*)workspace + scan, workspace_bytes - scan, stream, nullptr, nullptr, 0,
-                          words + B, 2, nullptr, &nearly_all);
+                          scale, words, 0, dense_ws, dense_bytes, stream, nullptr, nullptr, 0, flag, PREFIX_MOST, nullptr, &most);
       if (rc) return rc;
     }
     rc = attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,
-                        scale, words, 0, (char*)workspace + scan, workspace_bytes - scan, stream, nullptr, nullptr, 0,
-                        words + B, 1, nullptr, &fewer);
+                        scale, words, 0, dense_ws, dense_bytes, stream, nullptr, nullptr, 0, flag,
+                        dual ? PREFIX_FEWER : PREFIX_FEWER | PREFIX_MOST, nullptr, &fewer);
     if (rc) return rc;
-    p.gate = words + B;
-    p.gate_want = 0;
+    if (gather) {
+      uint16_t* const kc = (uint16_t*)((char*)workspace + lay.kc);
+      uint16_t* const vc = (uint16_t*)((char*)workspace + lay.vc);
+      AttnParams g = p;
+      g.gate = flag;
+      g.gate_mask = HOLES_FEWER | HOLES_MOST;
+      if (D == 128)
+        hipLaunchKernelGGL((gather_kept_keys_kernel<128>), dim3(nchunk, H, B), dim3(256), 0, st, g, (const uint8_t*)mask, p.ms_b, p.ms_k, nchunk,
+                           (const int32_t*)words, (const int32_t*)chunk_off, kc, vc);
+      else
+        hipLaunchKernelGGL((gather_kept_keys_kernel<64>), dim3(nchunk, H, B), dim3(256), 0, st, g, (const uint8_t*)mask, p.ms_b, p.ms_k, nchunk,
+                           (const int32_t*)words, (const int32_t*)chunk_off, kc, vc);
+      PA_CHECK_LAUNCH("key gather kernel");
+      const int64_t cs[3] = {(int64_t)H * Skv * D, (int64_t)Skv * D, D};
+      dual = stream_takes_key_counts(B, H, Sq, Skv, D, cs, cs, dense_bytes);
+      if (dual) {
+        rc = attn_fwd_dense(q, kc, vc, out, lse, dtype, B, H, Sq, Skv, D, q_strides, cs, cs, out_strides,
+                            scale, words, 0, dense_ws, dense_bytes, stream, nullptr, nullptr, 0, flag, HOLES_MOST, nullptr, &most);
+        if (rc) return rc;
+      }
+      return attn_fwd_dense(q, kc, vc, out, lse, dtype, B, H, Sq, Skv, D, q_strides, cs, cs, out_strides,
+                            scale, words, 0, dense_ws, dense_bytes, stream, nullptr, nullptr, 0, flag,
+                            dual ? HOLES_FEWER : HOLES_FEWER | HOLES_MOST, nullptr, &fewer);
+    }
+    p.gate = flag;
+    p.gate_mask = HOLES_FEWER | HOLES_MOST;
   }
   if (!any) {  // no rows, or no keys: the dense path writes what an empty softmax gives
     return attn_fwd_dense(q, k, v, out, lse, dtype, B, H, Sq, Skv, D, q_strides, k_strides, v_strides, out_strides,

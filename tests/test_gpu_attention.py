@@ -304,10 +304,13 @@ def test_long_launches_with_nearly_full_key_masks(cuda, rounds, tuning):
     the keys in every batch element -- a padded text prompt at the end of a video's tokens -- goes to the
     resident-workgroup kernel with the counts as per-batch key limits: pieces end at their batch element's last key,
     ranges of the tail that lie beyond it come out empty (with 6 rounds the last ranges are 32 tiles long and one
-    batch element drops 60).  A prefix that keeps less goes to the kernel with one workgroup per query tile, anything
-    else to the per-score kernel; which of the three runs is decided on the device.  Sampled rows of three heads
-    against the fp64 oracle; the nearly full case also against the same call with the resident-workgroup kernel
-    switched off, and bit for bit against a second call."""
+    batch element drops 60).  A prefix that keeps less goes to the kernel with one workgroup per query tile.  A mask
+    with holes -- one key missing, half of the keys at random, or the text padding of eight ranks' shards inside the
+    gathered sequence, as the reference's sequence-parallel HunyuanVideo adapter builds it
+    (context_parallel/diffusers_adapters/hunyuan_video.py:86-100) -- has its kept K and V rows gathered into dense
+    copies on which the same two kernels run.  Which launches run is decided on the device.  Sampled rows of three
+    heads against the fp64 oracle; the nearly full cases also against the same call with the resident-workgroup kernel
+    switched off, and bit for bit against a second call; attention_forward_sparse_kv gives the same output."""
     tuning("stream_dyn", rounds)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     B, H, D = 2, 8, 128
@@ -318,11 +321,19 @@ def test_long_launches_with_nearly_full_key_masks(cuda, rounds, tuning):
     heads = [0, 3, 7]
     rows = torch.cat([torch.arange(0, 150), torch.randint(0, Sq, (150,), generator=torch.Generator().manual_seed(2)), torch.arange(Sq - 150, Sq)])
     cases = [("nearly full", [Skv - 3, Skv - 64 * 60 - 5]),  # the second batch element is the one whose pieces make up the tail ("full", [Skv, Skv]), ("nearly full, whole tiles", [Skv - 13, Skv - 13 - 128]),
-             ("half", [Skv - 3, Skv // 2]), ("scattered", None)]
+             ("half", [Skv - 3, Skv // 2]), ("nearly full, one hole", None), ("random half", None), ("nearly full, interleaved padding", None)]
     for name, lens in cases:
-        if lens is None:
+        if name == "nearly full, one hole":
             m = torch.arange(Skv)[None, :] < torch.tensor([Skv - 3, Skv - 70])[:, None]
             m[1, 10] = False
+        elif name == "random half":
+            m = torch.rand(B, Skv, generator=torch.Generator().manual_seed(9)) < 0.5
+        elif name == "nearly full, interleaved padding":
+            shard, text = Skv // 8, 32  # per rank: latent tokens, then 32 text tokens; 100 / 37 of the 256 are valid
+            pos = torch.arange(Skv)
+            rank, off = pos // shard, pos % shard
+            text_index = rank * text + (off - (shard - text))
+            m = torch.stack([(off < shard - text) | (text_index < valid) | (pos >= 8 * shard) for valid in (100, 37)])
         else:
             m = torch.arange(Skv)[None, :] < torch.tensor(lens)[:, None]
         mask = m[:, None, None, :].to(cuda)
@@ -332,12 +343,33 @@ def test_long_launches_with_nearly_full_key_masks(cuda, rounds, tuning):
         assert torch.isfinite(lse).all() and torch.isfinite(out.float()).all()
         out2, lse2 = op(qd, kd, vd, mask)
         assert torch.equal(out2, out) and torch.equal(lse2, lse), name
+        assert torch.equal(torch.ops.para_attn.attention_forward_sparse_kv(qd, kd, vd, mask.expand(B, 1, Sq, Skv)), out), name
         if name.startswith("nearly"):
             tuning("stream", 0)
             out0, lse0 = op(qd, kd, vd, mask)
             tuning("stream", -1)
             assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
             assert not torch.equal(out0, out), "meant to run two different kernels"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_key_masks_with_holes_head_dim_64(cuda, dtype):
+    """head_dim 64, large enough (3e11 flop) for the kept keys of a mask with holes to be gathered: a random mask that
+    keeps 70 % and one that drops three keys, two batch elements, K in [B,S,H,D] memory; every head's sampled rows
+    against the fp64 oracle."""
+    B, H, Sq, Skv, D = 2, 6, 10000, 10007, 64
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=53, dtype=dtype)
+    qd, vd = q.to(cuda), v.to(cuda)
+    kd = k.to(cuda).transpose(1, 2).contiguous().transpose(1, 2)
+    rows = torch.cat([torch.arange(0, 100), torch.arange(Sq - 100, Sq)])
+    g = torch.Generator().manual_seed(6)
+    for name in ("random", "three holes"):
+        m = torch.rand(B, Skv, generator=g) < 0.7 if name == "random" else torch.ones(B, Skv, dtype=torch.bool)
+        m[0, 5] = m[1, 4000] = m[1, Skv - 1] = False
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), k.float().numpy(), v.float().numpy(), None, m[:, None, None, :].numpy())
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, m[:, None, None, :].to(cuda))
+        _check(out[:, :, rows.to(cuda)], lse[:, :, rows.to(cuda)], ref_out, ref_lse, f"head_dim 64, {name}, {dtype}")
+        assert torch.isfinite(out.float()).all()
 
 
 @pytest.mark.parametrize("D", [128, 64])

@@ -69,3 +69,38 @@ def test_graph_replays_match_eager(cuda, tuning):
         torch.cuda.synchronize()
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), f"replay {rep}: output {i} differs from the eager run"
+
+
+def test_graph_replays_of_a_masked_call_whose_mask_changes(cuda):
+    """A masked call large enough for the kept keys of a mask with holes to be gathered (3e11 flop), captured once and
+    replayed with a prefix mask, a mask with holes, a mask that keeps half of the keys at random and a prefix again:
+    which of the enqueued launches run is decided on the device at every replay."""
+    B, H, Sq, Skv, D = 1, 8, 9000, 9011, 128
+    q, k, v = (t.to(cuda) for t in inputs.qkv(B, H, Sq, Skv, D, seed=3))
+    mask = torch.ones(1, 1, 1, Skv, dtype=torch.bool, device=cuda)
+    op = torch.ops.para_attn.attention_forward_with_lse
+    op(q, k, v, mask)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        op(q, k, v, mask)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            captured = op(q, k, v, mask)
+    torch.cuda.synchronize()
+    g = torch.Generator().manual_seed(4)
+    masks = [torch.arange(Skv) < Skv - 100, (torch.arange(Skv) < Skv - 100) & (torch.arange(Skv) != 77), torch.rand(Skv, generator=g) < 0.5,
+             torch.arange(Skv) < 3000]
+    for rep, m in enumerate(masks):
+        mask.copy_(m[None, None, None, :])
+        q.copy_(torch.randn(q.shape, generator=g).bfloat16())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = op(q, k, v, mask)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), f"replay {rep}"
+        kept = m.nonzero()[:, 0].to(cuda)
+        ref = op(q, k[:, :, kept], v[:, :, kept])
+        assert (got[0].float() - ref[0].float()).abs().max().item() <= 2e-2 and (got[1] - ref[1]).abs().max().item() <= 1e-4, f"replay {rep}"
