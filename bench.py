@@ -145,12 +145,15 @@ def bench_attn(dev, steps, warmup):
 
 
 def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=(0,), traffic=None, causal=False, sets=1,
-                masked_keys=0):
+                masked_keys=0, shards=1):
     """One dense shape: timed, then sampled rows of the last timed output checked against torch's CPU SDPA.
     ``sets`` > 1: the calls rotate over that many copies of q, k, v at different addresses, so that a working set
     smaller than the 256 MB memory-side cache is not served from it call after call (in a model every call brings
     other tensors).  ``masked_keys`` > 0: the call passes a boolean key mask [1,1,1,Skv] that drops that many keys
-    at the end (a padded text prompt); flops and the check are those of the kept keys."""
+    (a padded text prompt of 256 tokens): at the end, or with ``shards`` > 1 where the padding lies when that many
+    ranks' [latent, text] shards have been gathered along the sequence, which is the mask the reference's
+    sequence-parallel HunyuanVideo adapter builds (context_parallel/diffusers_adapters/hunyuan_video.py:86-100);
+    flops and the check are those of the kept keys."""
     import torch
 
     from oracle import inputs
@@ -160,7 +163,14 @@ def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=
     op = torch.ops.para_attn.attention_forward_with_lse
     last = {}
     kept = Skv - masked_keys
-    mask = (torch.arange(Skv, device=dev) < kept)[None, None, None, :] if masked_keys else None
+    keep = None
+    if masked_keys:
+        pos = torch.arange(Skv)
+        shard, text = Skv // shards, 256 // shards
+        text_index = (pos // shard) * text + (pos % shard - (shard - text))  # position in the prompt, for text tokens
+        keep = (pos % shard < shard - text) | (text_index < 256 - masked_keys) | (pos >= shards * shard)
+        assert int(keep.sum()) == kept
+    mask = keep[None, None, None, :].to(dev) if masked_keys else None
 
     def call(i):
         qd, kd, vd = bufs[i % sets]
@@ -168,14 +178,17 @@ def _dense_case(dev, name, B, H, Sq, Skv, D, steps, warmup, seed=3, check_heads=
 
     t = _time_calls(call, steps, warmup)
     heads = sorted(set(list(check_heads) + [H - 1]))
-    checked = _check_rows(last["out"], last["lse"], q, k[:, :, :kept], v[:, :, :kept], heads, _sample_rows(Sq), name, causal=causal)
+    k_kept, v_kept = (k, v) if keep is None else (k[:, :, keep], v[:, :, keep])
+    checked = _check_rows(last["out"], last["lse"], q, k_kept, v_kept, heads, _sample_rows(Sq), name, causal=causal)
     flops = 4.0 * B * H * Sq * kept * D * (0.5 if causal else 1.0)  # causal: the kept half (Sq == Skv)
     nbytes = 2.0 * B * H * D * (2 * Sq + 2 * Skv) + 4.0 * B * H * Sq
     gbs = nbytes / (t["median"] * 1e-3) / 1e9
     more = {"traffic": TRAFFIC[traffic], "traffic_source": TRAFFIC_SOURCE} if traffic else {}
     if sets > 1:
         more["buffer_sets"] = sets
-    what = "attention_forward_with_lse" + (" is_causal" if causal else "") + (f" with a key mask that drops the last {masked_keys} keys" if masked_keys else "")
+    what = "attention_forward_with_lse" + (" is_causal" if causal else "")
+    if masked_keys:
+        what += f" with a key mask that drops {masked_keys} keys" + (" at the end" if shards == 1 else f" in the text parts of {shards} gathered shards")
     return _mfma(f"{name}: {what} q [{B},{H},{Sq},{D}] k,v [{B},{H},{Skv},{D}] bf16", flops, t,
                  bytes=nbytes, gbs=round(gbs, 1), frac_hbm=round(gbs / PEAK_HBM_GBS, 4), checked=checked, **more)
 
@@ -232,12 +245,15 @@ def bench_ring(dev, steps=6, warmup=3):
 
 def bench_shapes(dev, steps=10, warmup=5):
     """Further dense shapes: the headline shape with is_causal (flops of the kept half), the headline shape with the
-    key mask of a padded text prompt, and a head_dim 64 shape."""
+    key mask of a padded text prompt (as a prefix, and as it lies in the sequence gathered from 8 ranks), and a
+    head_dim 64 shape."""
     return {
         "headline_shape_causal": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=5,
                                              check_heads=(0, 1), causal=True, traffic="causal"),
         "headline_shape_text_mask": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=7,
                                                 check_heads=(0, 1), masked_keys=167, traffic="text_mask"),
+        "headline_shape_text_mask_8_shards": _dense_case(dev, "headline shape", 1, 3, 119056, 119056, 128, steps, warmup, seed=8,
+                                                         check_heads=(0, 1), masked_keys=167, shards=8),
         "head_dim_64": _dense_case(dev, "head_dim 64 (CogVideoX-like)", 1, 48, 17776, 17776, 64, steps, warmup, seed=6,
                                    check_heads=(0, 23), traffic="head_dim_64"),
     }

@@ -153,11 +153,19 @@ PA_API int pa_attn_fwd_lse_ws(const void* q, const void* k, const void* v, void*
  * device; where it keeps a prefix of the keys in every batch element the fast
  * dense kernels run with the counts as kv_len (long launches whose prefixes
  * keep at least 7/8 of the keys everywhere: the kernel with resident
- * workgroups, which plain dense calls use), otherwise, and for every other
- * mask, a kernel that reads the mask per score.  The choice is made on the
- * device: nothing is read back, so the call can be captured in a HIP graph.
+ * workgroups, which plain dense calls use).  Where it has holes (the mask of
+ * the reference's sequence-parallel HunyuanVideo adapter, whose text padding
+ * lies inside the gathered sequence:
+ * context_parallel/diffusers_adapters/hunyuan_video.py:86-100) and the call
+ * is one of 3e11 flop or more, the kept K and V rows are gathered into dense
+ * copies in the workspace, as the reference's attention_forward_sparse_kv
+ * does with index_select (ops/__init__.py:276-296), and the same kernels run
+ * on the copies.  Smaller calls with such a mask, and every other mask, run a
+ * kernel that reads the mask per score.  The choice is made on the device:
+ * nothing is read back, so the call can be captured in a HIP graph.
  * workspace: pa_attn_fwd_masked_workspace_bytes() bytes (16-byte aligned, any
- * contents); null or short is not an error: the per-score kernel runs.
+ * contents; from 3e11 flop on it includes the copies of K and V); null or
+ * short is not an error: the per-score kernel runs where there is no room.
  */
 PA_API int pa_attn_fwd_masked(const void* q, const void* k, const void* v, void* out, float* lse,
                        int dtype, int B, int H, int Sq, int Skv, int D,
