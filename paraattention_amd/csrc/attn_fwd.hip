@@ -26,7 +26,11 @@
 // Stands in for the aten flash/efficient/cuDNN forward kernels the reference
 // dispatches to (src/para_attn/ops/__init__.py:48-157) and, with a list of key
 // ranges per query segment, for the run loop of the reference's block-sparse
-// mode (src/para_attn/sparse_attn.py:209-240).
+// mode (src/para_attn/sparse_attn.py:209-240).  Boolean key masks are taken apart
+// on the device (key_mask_*_kernel) and served by the same kernels: in place with
+// per-batch key counts where they keep prefixes, on dense copies of the kept rows
+// (gather_kept_keys_kernel, the reference's attention_forward_sparse_kv,
+// src/para_attn/ops/__init__.py:248-299) where they have holes.
 
 #include <stdlib.h>
 #include <string.h>
