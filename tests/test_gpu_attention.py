@@ -352,6 +352,27 @@ def test_long_launches_with_nearly_full_key_masks(cuda, rounds, tuning):
             assert not torch.equal(out0, out), "meant to run two different kernels"
 
 
+@pytest.mark.parametrize("Sq,Skv", [(150, 333), (9000, 9011)])
+def test_key_masks_that_keep_nothing_in_one_batch_element(cuda, Sq, Skv):
+    """A key mask that drops every key of one batch element (out = 0, LSE = -inf there, the oracle's convention), as a
+    prefix of length 0 and, with a hole in the other element, as a mask with holes; at a small size (the per-score
+    kernel for the mask with holes) and at one where the kept keys are gathered."""
+    B, H, D = 2, 8, 128
+    q, k, v = inputs.qkv(B, H, Sq, Skv, D, seed=61)
+    qd, kd, vd = q.to(cuda), k.to(cuda), v.to(cuda)
+    rows = torch.cat([torch.arange(0, 60), torch.arange(Sq - 60, Sq)])
+    for holes in (False, True):
+        m = torch.ones(B, Skv, dtype=torch.bool)
+        m[0] = False
+        if holes:
+            m[1, 7] = False
+        ref_out, ref_lse = oattn.sdpa_lse_f64(q[:, :, rows].float().numpy(), k.float().numpy(), v.float().numpy(), None, m[:, None, None, :].numpy())
+        out, lse = torch.ops.para_attn.attention_forward_with_lse(qd, kd, vd, m[:, None, None, :].to(cuda))
+        _check(out[:, :, rows.to(cuda)], lse[:, :, rows.to(cuda)], ref_out, ref_lse, f"nothing kept in element 0, holes={holes}")
+        assert (out[0] == 0).all() and torch.isinf(lse[0]).all() and (lse[0] < 0).all()
+        assert torch.isfinite(out[1].float()).all() and torch.isfinite(lse[1]).all()
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_key_masks_with_holes_head_dim_64(cuda, dtype):
     """head_dim 64, large enough (3e11 flop) for the kept keys of a mask with holes to be gathered: a random mask that
