@@ -61,7 +61,7 @@ PA_API const char* pa_last_error(void);
  *   "stream_even"  PARAATTN_STREAM_EVEN=0|1 that kernel's tail cut into shares that begin at the same keys / into equal ranges, -1 = by size
  *   "stream_dyn"   PARAATTN_STREAM_DYN=0|2..6  that kernel's tail in equal ranges, one per workgroup / in that many rounds of ever
  *                                           shorter ranges which the workgroups draw from a counter as they run out of work (so
- *                                           that faster compute units take more), wherever two rounds fit; -1 = 4 rounds from 1024
+ *                                           that faster compute units take more), wherever two rounds fit; -1 = 4 rounds from 2048
  *                                           key-tile steps per workgroup on.  Needs 4x the workspace of equal ranges; a call whose
  *                                           workspace is smaller gets equal ranges.  Results do not depend on who drew what.
  *   "stream_solo"  PARAATTN_STREAM_SOLO=1   test aid: a launch all of whose pieces are cut into drawn ranges (fewer pieces than

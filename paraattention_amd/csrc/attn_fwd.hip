@@ -4089,16 +4089,18 @@ static bool plan_stream(AttnParams& p, int D, const KeySegs* segs, size_t ws_ava
   // on the keys, but leave workgroups idle; measured slower or equal at every shape from 3000 to 119056 keys
   const int ev = tuning().stream_even;
   const bool even = ev != 0;
-  // Rounds of ever shorter ranges that go to whoever asks first (StreamPlan::next_range), from 1024 key-tile steps per
+  // Rounds of ever shorter ranges that go to whoever asks first (StreamPlan::next_range), from 2048 key-tile steps per
   // workgroup on.  Workgroups given equal shares finish up to 7 % apart (some XCDs are slower than others, by box);
-  // drawn ranges bring that below 1 % and take 1.7 .. 2.9 % off the time of launches of 2.5 ms and more (119056 keys,
-  // Wan self-attention, a ring sweep, 16k tokens x 40 heads), but their 4 G partial results cost about 35 us to write
-  // and fold, which shorter launches do not earn back (measured +1 .. +8 % from 0.4 to 1.2 ms).
+  // drawn ranges bring that below 1 % and take 1.7 .. 2.9 % off the time of launches of 4 ms and more (119056 keys,
+  // Wan self-attention, a ring sweep, 16k tokens x 40 heads) on boxes with such a spread, 0 .. 1 % on boxes whose XCDs
+  // run alike.  Their 4 G partial results cost about 35 us to write and fold, which shorter launches do not earn
+  // back (+1 .. +8 % from 0.4 to 1.2 ms on any box; between 1024 and 2048 steps -0.6 .. -1 % on a box with the spread,
+  // +0.6 .. +1.2 % on one without).
   int dyn = 0;
   if (allow_drawn && even && !tuning().no_split && (sizing || ws_avail > 0)) {
     const int want_dyn = tuning().stream_dyn;
     if (want_dyn > 1) dyn = want_dyn;
-    else if (want_dyn < 0 && (int64_t)P * L >= (int64_t)1024 * st.G) dyn = 4;
+    else if (want_dyn < 0 && (int64_t)P * L >= (int64_t)2048 * st.G) dyn = 4;
   }
   int p_tail = P - st.R * st.G;
   if (dyn > 1) {

@@ -349,7 +349,8 @@ def test_long_launches_with_nearly_full_key_masks(cuda, rounds, tuning):
             out0, lse0 = op(qd, kd, vd, mask)
             tuning("stream", -1)
             assert (out.float() - out0.float()).abs().max().item() <= 2e-2 and (lse - lse0).abs().max().item() <= 1e-4
-            assert not torch.equal(out0, out), "meant to run two different kernels"
+            if rounds > 0:  # (whole pieces come out bit-equal from both kernels: the same tiles in the same order)
+                assert not torch.equal(out0, out), "meant to run two different kernels"
 
 
 @pytest.mark.parametrize("Sq,Skv", [(150, 333), (9000, 9011)])
@@ -532,7 +533,7 @@ def test_resident_workgroup_kernel(cuda, even, bound, wave_rows, tuning):
 @pytest.mark.parametrize("wave_rows", [32, 64])
 def test_resident_workgroups_draw_their_tail_ranges(cuda, rounds, wave_rows, tuning):
     """The resident-workgroup kernel with its tail cut into rounds of ever shorter ranges that the workgroups draw
-    from a counter as they run out of work (by itself the planner does that from 1024 key-tile steps per workgroup
+    from a counter as they run out of work (by itself the planner does that from 2048 key-tile steps per workgroup
     on; forced here at sizes the oracle can follow): fewer pieces than workgroups, a few pieces beyond a whole round,
     and exactly two rounds of pieces (the plan then gives up a round of whole pieces to have a tail), ragged query
     and key ends, both dtypes.  Sampled rows of three heads against the fp64 oracle; the whole output against the
@@ -652,7 +653,7 @@ def test_drawn_ranges_random_configurations(cuda, tuning):
 
 def test_planner_draws_ranges_for_long_launches_only(cuda, tuning):
     """What the planner asks of the workspace says which plan it took: four rounds of ranges (4 x compute units x two
-    partial results, and the counter's 256 bytes) from 1024 key-tile steps per workgroup on, at most one range per
+    partial results, and the counter's 256 bytes) from 2048 key-tile steps per workgroup on, at most one range per
     workgroup below."""
     import ctypes
 
