@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # rocprofv3 --pmc runs of `bench.py --only <kernel>` (scale factors from a 1 GiB copy).  These counters cannot be
 # read from inside this process; the figures are those of the summary named in TRAFFIC_SOURCE, not of this run.
 TRAFFIC = {"attn": 1.005e10, "merge": 4.773e8, "fbcache": 6.710e8, "taylorseer": 1.677e9, "sparse": 8.940e9,
-           "flux": 3.039e8, "ring_sweep": 1.234e10, "ring_sweep_per_block": 1.436e10, "wan_self": 3.797e9, "wan_cross": 7.013e8,
+           "flux": 3.039e8, "ring_sweep": 1.234e10, "ring_sweep_per_block": 1.509e10, "wan_self": 3.797e9, "wan_cross": 7.013e8,
            "causal": 5.153e9, "text_mask": 1.005e10, "head_dim_64": 2.438e9}
 TRAFFIC_SOURCE = "profiles/kernels_bench_workloads.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the same command)"
 
